@@ -1,0 +1,140 @@
+/*
+ * yamoe_hip.h — C ABI of libyamoe_hip.so: the MI355X (gfx950) expert-layer path.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream handle
+ * (passed as void* so that this header needs no HIP include).  Nothing here
+ * allocates, frees or synchronises: callers bring the output buffers and one
+ * workspace whose size the matching *_workspace_bytes() call returns.  All work
+ * is enqueued on `stream` and the call returns at once.
+ *
+ * Return value: 0 on success, a negative YAMOE_E_* code on a rejected argument,
+ * a positive hipError_t if a launch failed.  yamoe_last_error() gives the text
+ * of the last failure on the calling thread.
+ *
+ * Citations name the file:line of drbh/yamoe that each entry point replaces.
+ */
+#ifndef YAMOE_HIP_H
+#define YAMOE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define YAMOE_ABI_VERSION 1
+
+/* element type of activations, weights, biases and routing weights */
+enum { YAMOE_F32 = 0, YAMOE_F16 = 1, YAMOE_BF16 = 2 };
+
+enum {
+  YAMOE_E_ARG = -1,       /* bad size / null pointer / unsupported shape */
+  YAMOE_E_WORKSPACE = -2, /* workspace too small */
+  YAMOE_E_DTYPE = -3      /* unknown dtype */
+};
+
+/* Shape of one experts() call.  Mirrors the integer arguments and tensor sizes
+ * of experts_cuda (csrc/moe.cpp:45-96). */
+typedef struct yamoe_problem {
+  int32_t T;         /* tokens (rows of hidden_states) */
+  int32_t K;         /* top_k: experts per token */
+  int32_t E;         /* num_experts */
+  int32_t H;         /* hidden size */
+  int32_t I;         /* intermediate size; gate_up_proj is [E,H,2I], down_proj is [E,I,H] */
+  int32_t capacity;  /* expert_capacity: assignments ranked >= capacity inside their expert are dropped */
+  int32_t dtype;     /* YAMOE_F32 / YAMOE_F16 / YAMOE_BF16 */
+  int32_t idx_i64;   /* router_indices element type: 1 = int64, 0 = int32 */
+  int32_t rw_cols;   /* columns of routing_weights: E (dense [T,E]) or K (per slot [T,K]) */
+} yamoe_problem;
+
+int yamoe_abi_version(void);
+const char *yamoe_last_error(void);
+
+/* ---- routing: stable sort of (token,slot) assignments by expert -------------
+ * Replaces sort_cuda (csrc/sort.cu:61-91) + bincount_cumsum_cuda
+ * (csrc/bincount_cumsum.cu:58-97) as called from csrc/moe.cpp:141-144.
+ *   router_indices [N]  int32 or int64 expert id per flat slot t*K+k (N = T*K)
+ *   sorted_expert  [N]  expert ids in non-decreasing order
+ *   sorted_idx     [N]  flat slot of each sorted position; ties keep slot order (stable)
+ *   counts         [E]  assignments per expert
+ *   offsets        [E+1] exclusive prefix sum of counts; offsets[E] = number of valid ids
+ *   inv_pos        [N]  sorted position of each flat slot, or -1 when the slot is
+ *                       dropped (rank inside its expert >= capacity, or id outside [0,E))
+ * Ids outside [0,E) sort after every valid expert. */
+size_t yamoe_route_workspace_bytes(int32_t N, int32_t E);
+int yamoe_route(const void *router_indices, int32_t idx_i64, int32_t N, int32_t E,
+                int32_t capacity, int32_t *sorted_expert, int32_t *sorted_idx,
+                int32_t *counts, int32_t *offsets, int32_t *inv_pos, void *workspace,
+                size_t workspace_bytes, void *stream);
+
+/* ---- token permute: expert-contiguous row gather -----------------------------
+ * Replaces gather_cuda (csrc/gather.cu:68-109) without the padded [E,C,H] layout:
+ *   x_perm[p,:] = x[sorted_idx[p] / K, :]   for every sorted position p < N. */
+int yamoe_permute(const void *x, const int32_t *sorted_idx, void *x_perm, int32_t N,
+                  int32_t K, int32_t H, int32_t dtype, void *stream);
+
+/* ---- routing-weighted combine -------------------------------------------------
+ * Replaces at::gather_out + index_select_out_cuda + scatter_cuda
+ * (csrc/moe.cpp:190-220, csrc/index_select.cu:18-51, csrc/scatter.cu:110-147):
+ *   out[t,:] = sum_k w(t,k) * y_perm[inv_pos[t*K+k],:]   (dropped slots skipped)
+ * with w(t,k) = routing_weights[t, router_indices[t,k]] when rw_cols == E and
+ * routing_weights[t,k] when rw_cols == K.  Sum in fp32 in slot order, one
+ * rounding; no atomics, `out` needs no zero fill.  routing_weights == NULL
+ * means weight 1 (the backward of the permute, csrc/experts_backward.cu:92-124). */
+int yamoe_combine(const void *y_perm, const int32_t *inv_pos, const void *router_indices,
+                  int32_t idx_i64, const void *routing_weights, int32_t rw_cols, void *out,
+                  int32_t T, int32_t K, int32_t E, int32_t H, int32_t dtype, void *stream);
+
+/* ---- expert GEMMs --------------------------------------------------------------
+ * Replace batch_mm (csrc/batch_mm.cu:7-31) plus the ATen bias / clamped-SwiGLU
+ * chain (csrc/moe.cpp:161-187) on ragged expert groups (no padding):
+ *   gate_up: act[p, j] = (clamp(U,-7,7)+1) * g*sigmoid(1.702 g), g = min(G,7),
+ *            G = x_p . Wgu[e][:,2j] + bgu[e][2j],  U = x_p . Wgu[e][:,2j+1] + bgu[e][2j+1]
+ *            with x_p = x[sorted_idx[p]/K] gathered on the fly (x is the un-permuted [T,H]).
+ *            If pre_act != NULL the biased pre-activations [N,2I] are stored too.
+ *   down:    y_perm[p,:] = act[p,:] . Wd[e] + bd[e]
+ * Rows p with rank >= capacity inside their expert are not computed.
+ * `schedule` is the workspace region filled by yamoe_build_schedule: experts with
+ * 1..stream_max_rows kept rows (at most 16; 16-bit dtypes only, pass 0 for fp32) are
+ * listed for the weight-streaming kernel, the others are cut into 256-row MFMA tiles.
+ * yamoe_gate_up / yamoe_down launch both kernels; each walks its own list. */
+size_t yamoe_schedule_bytes(int32_t N, int32_t E);
+int yamoe_build_schedule(const int32_t *counts, const int32_t *offsets, int32_t N, int32_t E,
+                         int32_t capacity, int32_t stream_max_rows, void *schedule,
+                         size_t schedule_bytes, void *stream);
+int yamoe_gate_up(const void *x, const int32_t *sorted_idx, const void *gate_up_proj,
+                  const void *gate_up_proj_bias, void *act, void *pre_act, const void *schedule,
+                  int32_t N, int32_t K, int32_t E, int32_t H, int32_t I, int32_t dtype,
+                  void *stream);
+int yamoe_down(const void *act, const void *down_proj, const void *down_proj_bias, void *y_perm,
+               const void *schedule, int32_t N, int32_t E, int32_t H, int32_t I, int32_t dtype,
+               void *stream);
+
+/* ---- the whole forward: experts_cuda (csrc/moe.cpp:45-223) ------------------- */
+size_t yamoe_experts_workspace_bytes(const yamoe_problem *p);
+int yamoe_experts_forward(const yamoe_problem *p, const void *hidden_states,
+                          const void *router_indices, const void *routing_weights,
+                          const void *gate_up_proj, const void *gate_up_proj_bias,
+                          const void *down_proj, const void *down_proj_bias, void *out,
+                          void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- the whole backward: experts_backward_cuda (csrc/experts_backward.cu:126-341)
+ * Outputs (all fully written, caller need not zero them):
+ *   d_hidden [T,H], d_routing [T,rw_cols] (zero outside the selected experts),
+ *   d_gate_up_proj [E,H,2I], d_gate_up_proj_bias [E,2I], d_down_proj [E,I,H],
+ *   d_down_proj_bias [E,H].  grad_out is [T,H]. */
+size_t yamoe_experts_backward_workspace_bytes(const yamoe_problem *p);
+int yamoe_experts_backward(const yamoe_problem *p, const void *grad_out,
+                           const void *hidden_states, const void *router_indices,
+                           const void *routing_weights, const void *gate_up_proj,
+                           const void *gate_up_proj_bias, const void *down_proj,
+                           const void *down_proj_bias, void *d_hidden, void *d_routing,
+                           void *d_gate_up_proj, void *d_gate_up_proj_bias, void *d_down_proj,
+                           void *d_down_proj_bias, void *workspace, size_t workspace_bytes,
+                           void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* YAMOE_HIP_H */

@@ -1,0 +1,238 @@
+"""CPU oracle for the yamoe expert-layer path.  TEST INFRASTRUCTURE ONLY.
+
+This module restates, on the CPU, what drbh/yamoe computes on the `experts` / `experts_backward`
+path.  It exists to check the HIP kernels; nothing in the product (yamoe_amd/) imports it, and only
+tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may call it.
+
+Integer work (routing) is numpy; floating-point work is torch on the CPU (the reference's own
+language: its oracles are plain torch).  Each function cites the reference lines it follows
+(paths relative to the drbh/yamoe tree).
+
+Pinning (what each function is checked against in tests/test_oracle.py, none of which retypes the
+formula under test):
+  route                 brute-force O(N^2) rank count on small inputs, numpy stable argsort,
+                        permutation / monotonicity / stability invariants
+  glu                   hand-computed known answers (tests/golden/glu_kat.json, made with Python's
+                        math module in tests/golden/make_glu_kat.py), limits G=0, U=-1, saturation
+  experts_loop          agrees with experts_dense (an independent formulation: all experts on all
+                        tokens, dense weights) in fp64; special cases that reduce to one matmul
+                        (single expert), to a row copy (interleaved-identity weights), to a
+                        bias-only closed form (zero weights), and linearity in routing weights
+  experts_capacity      brute-force per-slot Python loops on tiny inputs; equals experts_loop when
+                        capacity >= max load
+  experts_backward      torch.autograd.gradcheck of experts_capacity in fp64 (finite differences),
+                        and agreement between autograd and the closed-form experts_backward_closed
+The reference ships no golden vectors or known-answer tests for this path (its tests directory is
+git-ignored), so no reference-held fixture exists to check against; no function here is
+"parity unpinned" in the sense of lacking an independent check.
+"""
+import numpy as np
+import torch
+
+GLU_LIMIT = 7.0   # csrc/moe.cpp:175; reference.py:16
+GLU_ALPHA = 1.702  # csrc/moe.cpp:179; reference.py:15
+
+
+# ------------------------------------------------------------------------------------------------
+# routing
+# ------------------------------------------------------------------------------------------------
+def route(router_indices, num_experts, capacity):
+    """Stable sort of flat (token, slot) assignments by expert id.
+
+    Follows sort_tokens_by_expert (torch-ext/yamoe/vendored/yamoe_ref.py:38-43), the radix sort it
+    stands for (csrc/sort.cu:17-59: keys = expert ids, values = iota, stable) and
+    bincount + cumsum (csrc/bincount_cumsum.cu:7-56).  Ids outside [0, E) sort last and are dropped.
+
+    Returns dict of int32 arrays: sorted_expert [N], sorted_idx [N], counts [E], offsets [E+1]
+    (exclusive; offsets[E] = number of valid ids), bins [E] (inclusive cumsum, the reference's
+    `bins`), inv_pos [N] (sorted position of each flat slot, -1 if dropped by the capacity rule:
+    rank inside its expert >= capacity, binned_gather yamoe_ref.py:10).
+    """
+    ids = np.asarray(router_indices).reshape(-1).astype(np.int64)
+    N, E = ids.shape[0], int(num_experts)
+    key = np.where((ids < 0) | (ids >= E), E, ids)
+    order = np.argsort(key, kind="stable").astype(np.int32)
+    counts_all = np.bincount(key, minlength=E + 1).astype(np.int64)
+    counts = counts_all[:E].astype(np.int32)
+    offsets = np.zeros(E + 1, dtype=np.int32)
+    offsets[1:] = np.cumsum(counts_all[:E])
+    bins = np.cumsum(counts).astype(np.int32)
+    sorted_expert = ids[order].astype(np.int32)
+    inv_pos = np.full(N, -1, dtype=np.int32)
+    pos = np.arange(N, dtype=np.int64)
+    skey = key[order]
+    valid = skey < E
+    rank = pos - offsets[np.minimum(skey, E - 1)]
+    kept = valid & (rank < capacity)
+    inv_pos[order[kept]] = pos[kept].astype(np.int32)
+    return dict(sorted_expert=sorted_expert, sorted_idx=order, counts=counts, offsets=offsets, bins=bins,
+                inv_pos=inv_pos)
+
+
+# ------------------------------------------------------------------------------------------------
+# activation
+# ------------------------------------------------------------------------------------------------
+def glu(gate_up):
+    """Clamped SwiGLU on interleaved columns: gate = even, up = odd.
+    reference.py:49-54 (build/torch28-cxx11-cu129-x86_64-linux/yamoe/reference.py); csrc/moe.cpp:164-180."""
+    gate, up = gate_up[..., ::2], gate_up[..., 1::2]
+    gate = gate.clamp(min=None, max=GLU_LIMIT)
+    up = up.clamp(min=-GLU_LIMIT, max=GLU_LIMIT)
+    return (up + 1) * (gate * torch.sigmoid(gate * GLU_ALPHA))
+
+
+# ------------------------------------------------------------------------------------------------
+# forward
+# ------------------------------------------------------------------------------------------------
+def experts_loop(hidden, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
+                 down_proj_bias, compute_dtype=None):
+    """Loop over the experts that were hit; the path the reference takes in training mode and on the
+    CPU (reference.py:38-59; torch-ext/yamoe/vendored/gpt_oss_mlp.py:57-92).  routing_weights is the
+    dense [T,E] matrix.  No capacity.  Every op runs in `compute_dtype` (default: the input dtype,
+    as the reference does) and the result is accumulated in that dtype with index_add_."""
+    dt = compute_dtype or hidden.dtype
+    x = hidden.reshape(-1, hidden.shape[-1]).to(dt)
+    rw = routing_weights.to(dt)
+    wgu, bgu, wd, bd = (t.to(dt) for t in (gate_up_proj, gate_up_proj_bias, down_proj, down_proj_bias))
+    E = rw.shape[1]
+    out = torch.zeros_like(x)
+    mask = torch.nn.functional.one_hot(router_indices.long(), num_classes=E).permute(2, 1, 0)  # [E,K,T]
+    hit = torch.greater(mask.sum(dim=(-1, -2)), 0).nonzero()
+    for e in hit[:, 0].tolist():
+        _, token_idx = torch.where(mask[e])
+        cur = x[token_idx]
+        gu = cur @ wgu[e] + bgu[e]
+        y = glu(gu) @ wd[e] + bd[e]
+        out.index_add_(0, token_idx, (y * rw[token_idx, e, None]).to(dt))
+    return out
+
+
+def experts_dense(hidden, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj, down_proj_bias,
+                  compute_dtype=None):
+    """Every expert on every token, weighted by the dense routing matrix and summed over experts:
+    the reference's inference path (reference.py:60-72).  Equal to experts_loop whenever the dense
+    weights are zero outside the selected experts."""
+    dt = compute_dtype or hidden.dtype
+    x = hidden.reshape(-1, hidden.shape[-1]).to(dt)
+    rw = routing_weights.to(dt)
+    E = rw.shape[1]
+    xe = x.repeat(E, 1).view(E, -1, x.shape[-1])
+    gu = torch.bmm(xe, gate_up_proj.to(dt)) + gate_up_proj_bias.to(dt)[..., None, :]
+    y = torch.bmm(glu(gu), down_proj.to(dt)) + down_proj_bias.to(dt)[..., None, :]
+    y = y * rw.transpose(0, 1)[..., None]
+    return y.sum(dim=0)
+
+
+def experts_capacity(hidden, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
+                     down_proj_bias, capacity, compute_dtype=None):
+    """The op's own semantics (csrc/moe.cpp:138-220 as restated by binned_experts_ref,
+    torch-ext/yamoe/vendored/yamoe_ref.py:46-82): assignments are sorted by expert (stable), the first
+    `capacity` of each expert are computed, the rest contribute nothing.  routing_weights may be the
+    dense [T,E] matrix or per-slot [T,K].  Differentiable with torch.autograd (the routing is
+    integer work done outside the graph).  Accumulation over a token's slots is a plain sum in
+    `compute_dtype`."""
+    dt = compute_dtype or hidden.dtype
+    x = hidden.reshape(-1, hidden.shape[-1]).to(dt)
+    T, K = router_indices.shape
+    E = gate_up_proj.shape[0]
+    r = route(router_indices.detach().cpu().numpy(), E, capacity)
+    rw = routing_weights.to(dt)
+    if rw.shape[1] == E:
+        safe = router_indices.long().clamp(0, E - 1)
+        w_sel = torch.gather(rw, 1, safe).reshape(-1)
+    else:
+        w_sel = rw.reshape(-1)
+    wgu, bgu, wd, bd = (t.to(dt) for t in (gate_up_proj, gate_up_proj_bias, down_proj, down_proj_bias))
+    out = torch.zeros_like(x)
+    for e in range(E):
+        n = min(int(r["counts"][e]), int(capacity))
+        if n <= 0:
+            continue
+        first = int(r["offsets"][e])
+        flat = torch.from_numpy(r["sorted_idx"][first:first + n].astype(np.int64))
+        tok = flat // K
+        gu = x[tok] @ wgu[e] + bgu[e]
+        y = glu(gu) @ wd[e] + bd[e]
+        out = out.index_add(0, tok, y * w_sel[flat, None])
+    return out
+
+
+# ------------------------------------------------------------------------------------------------
+# backward
+# ------------------------------------------------------------------------------------------------
+def experts_backward(grad_out, hidden, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias,
+                     down_proj, down_proj_bias, capacity, compute_dtype=torch.float32):
+    """Gradients of experts_capacity by torch.autograd: (d_hidden, d_routing, d_gate_up_proj,
+    d_gate_up_proj_bias, d_down_proj, d_down_proj_bias), the return order of experts_backward_cuda
+    (csrc/experts_backward.cu:340) and of _ExpertsFn.backward (torch-ext/yamoe/layers.py:50-100).
+    d_routing has the shape of routing_weights and is zero outside the selected experts, which is
+    what autograd through the loop path gives (reference.py:57)."""
+    leaves = [t.detach().to(compute_dtype).clone().requires_grad_(True)
+              for t in (hidden, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj, down_proj_bias)]
+    out = experts_capacity(leaves[0], router_indices, leaves[1], leaves[2], leaves[3], leaves[4], leaves[5],
+                           capacity, compute_dtype)
+    grads = torch.autograd.grad(out, leaves, grad_out.reshape(out.shape).to(compute_dtype), allow_unused=True)
+    return tuple(torch.zeros_like(l) if g is None else g for g, l in zip(grads, leaves))
+
+
+def experts_backward_closed(grad_out, hidden, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias,
+                            down_proj, down_proj_bias, capacity, compute_dtype=torch.float64):
+    """Closed-form backward, one expert at a time, following the formulas of
+    csrc/experts_backward.cu:231-311 (with the routing gradient placed at [t, expert] once, not
+    permuted twice as :261-264 does)."""
+    dt = compute_dtype
+    x = hidden.reshape(-1, hidden.shape[-1]).to(dt)
+    gy = grad_out.reshape(x.shape).to(dt)
+    T, K = router_indices.shape
+    E = gate_up_proj.shape[0]
+    r = route(router_indices.detach().cpu().numpy(), E, capacity)
+    rw = routing_weights.to(dt)
+    dense = rw.shape[1] == E
+    wgu, bgu, wd, bd = (t.to(dt) for t in (gate_up_proj, gate_up_proj_bias, down_proj, down_proj_bias))
+    d_x, d_rw = torch.zeros_like(x), torch.zeros_like(rw)
+    d_wgu, d_bgu, d_wd, d_bd = (torch.zeros_like(t) for t in (wgu, bgu, wd, bd))
+    for e in range(E):
+        n = min(int(r["counts"][e]), int(capacity))
+        if n <= 0:
+            continue
+        first = int(r["offsets"][e])
+        flat = torch.from_numpy(r["sorted_idx"][first:first + n].astype(np.int64))
+        tok, slot = flat // K, flat % K
+        w = rw[tok, e] if dense else rw[tok, slot]
+        xe = x[tok]
+        pre = xe @ wgu[e] + bgu[e]
+        G, U = pre[:, ::2], pre[:, 1::2]
+        g = G.clamp(max=GLU_LIMIT)
+        u = U.clamp(-GLU_LIMIT, GLU_LIMIT)
+        s = torch.sigmoid(GLU_ALPHA * g)
+        a = g * s
+        h = (u + 1) * a
+        ye = h @ wd[e] + bd[e]
+        g_ye = gy[tok] * w[:, None]
+        dots = (gy[tok] * ye).sum(-1)
+        if dense:
+            d_rw[tok, e] += dots
+        else:
+            d_rw[tok, slot] += dots
+        d_bd[e] = g_ye.sum(0)
+        g_h = g_ye @ wd[e].T
+        d_wd[e] = h.T @ g_ye
+        d_u = g_h * a * ((U >= -GLU_LIMIT) & (U <= GLU_LIMIT))
+        d_g = g_h * (u + 1) * (s + g * s * (1 - s) * GLU_ALPHA) * (G <= GLU_LIMIT)
+        d_pre = torch.stack([d_g, d_u], dim=-1).reshape(pre.shape)
+        d_bgu[e] = d_pre.sum(0)
+        d_wgu[e] = xe.T @ d_pre
+        d_x.index_add_(0, tok, d_pre @ wgu[e].T)
+    return d_x, d_rw, d_wgu, d_bgu, d_wd, d_bd
+
+
+# ------------------------------------------------------------------------------------------------
+# metrics (definitions of compare_example.py:207-214)
+# ------------------------------------------------------------------------------------------------
+def rel_l2(a, b):
+    a, b = a.double().cpu(), b.double().cpu()
+    return float((a - b).norm() / b.norm().clamp_min(1e-30))
+
+
+def max_abs(a, b):
+    return float((a.double().cpu() - b.double().cpu()).abs().max()) if a.numel() else 0.0

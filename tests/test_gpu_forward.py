@@ -1,0 +1,126 @@
+"""experts() forward through the torch op (-> C ABI -> HIP kernels) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import yamoe_oracle as O
+from tests.util import REL_L2_TOL, args, oracle_forward, report, to_dev
+from yamoe_amd.workloads import make_config, make_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def run_op(d, capacity, gpu):
+    import yamoe_amd
+    g = to_dev(d, gpu)
+    E, K = d["gate_up_proj"].shape[0], d["router_indices"].shape[1]
+    out = yamoe_amd.experts(*args(g), capacity, E, K)
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+SMALL = [
+    # T, H, I, E, K  -- chosen to hit: streaming path only, MFMA tiles only, both, ragged edges
+    (8, 64, 64, 4, 2),        # a few rows per expert: weight-streaming kernel
+    (64, 128, 96, 16, 4),     # I != H, streaming
+    (700, 64, 64, 2, 1),      # 350 rows per expert: MFMA tiles with a partial second tile
+    (1024, 256, 192, 4, 2),   # several column tiles? no: one; K slabs > 1
+    (300, 320, 136, 3, 2),    # N and K not multiples of the tile sizes
+    (513, 520, 264, 5, 3),    # more than one column tile for gate_up (2I = 528 > 256), K = 520 not /64
+    (2000, 64, 64, 64, 2),    # mix: some experts <= 16 rows, some above
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("T,H,I,E,K", SMALL)
+def test_forward_small(gpu, dtype, T, H, I, E, K):
+    print("forward_small", dtype, T, H, I, E, K, flush=True)
+    d = make_inputs(T, H, I, E, K, dtype, seed=T + H, w_std=0.05, bias_std=0.1, zipf=0.8 if E >= 16 else 0.0)
+    got = run_op(d, T, gpu)
+    want = oracle_forward(d, T)
+    r = report("fwd", got, want, REL_L2_TOL[dtype])
+    assert r < REL_L2_TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_forward_capacity_drop_and_slot_weights(gpu, dtype):
+    T, H, I, E, K = 400, 64, 64, 4, 2
+    d = make_inputs(T, H, I, E, K, dtype, seed=11, w_std=0.05, bias_std=0.1, zipf=1.0)
+    for C in (0, 7, 60, 150):
+        print("capacity", dtype, C, flush=True)
+        got = run_op(d, C, gpu)
+        want = oracle_forward(d, C)
+        if C == 0:
+            assert torch.all(got == 0)
+        else:
+            assert report("cap%d" % C, got, want, REL_L2_TOL[dtype]) < REL_L2_TOL[dtype]
+    # [T,K] routing weights and int32 indices are accepted and give the same bits
+    base = run_op(d, 60, gpu)
+    d2 = dict(d)
+    d2["routing_weights"] = torch.gather(d["routing_weights"], 1, d["router_indices"])
+    d2["router_indices"] = d["router_indices"].to(torch.int32)
+    assert torch.equal(run_op(d2, 60, gpu), base)
+
+
+def test_forward_special_cases(gpu):
+    """Structure checks that do not depend on the oracle's matmul: one-hot routing returns the
+    expert's row, zero weights reduce to the bias closed form, an unused expert changes nothing."""
+    dtype = torch.float32
+    T, H, I, E, K = 96, 64, 64, 4, 1
+    d = make_inputs(T, H, I, E, K, dtype, seed=3, w_std=0.05, bias_std=0.1)
+    d["routing_weights"] = torch.zeros(T, E).scatter_(1, d["router_indices"], 1.0)
+    d["gate_up_proj"].zero_()
+    got = run_op(d, T, gpu)
+    per_e = torch.stack([O.glu(d["gate_up_proj_bias"][e][None])[0] @ d["down_proj"][e] + d["down_proj_bias"][e]
+                         for e in range(E)])
+    want = per_e[d["router_indices"][:, 0]]
+    assert O.rel_l2(got, want) < 1e-5
+    # determinism: bitwise equal on a second run
+    assert torch.equal(run_op(d, T, gpu), got)
+
+
+def test_forward_gptoss20b_full(gpu):
+    """The GPT-OSS-20B shaped layer at full size against the fp32 oracle on the bf16 inputs."""
+    d, c = make_config("gptoss20b", seed=0)
+    got = run_op(d, c["T"], gpu)
+    want = oracle_forward(d, c["T"])
+    assert report("gptoss20b", got, want, 1e-2) < 1e-2
+    # size-independent properties: linear in the routing weights, and a token routed with all its
+    # weight on one expert equals that expert alone
+    d2 = dict(d)
+    d2["routing_weights"] = (d["routing_weights"].float() * 0.5).to(torch.bfloat16)  # exact scaling in bf16
+    half = run_op(d2, c["T"], gpu)
+    assert O.rel_l2(half.float() * 2, got.float()) < 1e-2
+
+
+def test_forward_decode_full_rows(gpu):
+    """Decode regime at the real expert shape (fewer experts to keep host generation short)."""
+    d = make_inputs(64, 2880, 2880, 32, 4, torch.bfloat16, seed=5)
+    counts = np.bincount(d["router_indices"].numpy().ravel(), minlength=32)
+    assert counts.max() <= 16  # every expert takes the streaming path
+    got = run_op(d, 64, gpu)
+    want = oracle_forward(d, 64)
+    assert report("decode", got, want, 1e-2) < 1e-2
+
+
+def test_forward_readme_shape_fp32(gpu):
+    """README shape (fp32, randn weights, heavy clamp saturation), two experts' worth of the 8 to
+    bound the oracle's time: rel-L2 <= 1e-5."""
+    d = make_inputs(4096, 2880, 2880, 2, 2, torch.float32, seed=42, w_std=1.0, bias_std=0.0, renorm=False)
+    got = run_op(d, 4096, gpu)
+    want = oracle_forward(d, 4096, compute_dtype=torch.float64)
+    assert report("readme-fp32", got, want, 1e-5) < 1e-5
+
+
+def test_op_rejects_bad_arguments(gpu):
+    import yamoe_amd
+    d = to_dev(make_inputs(8, 64, 64, 4, 2, torch.bfloat16), gpu)
+    a = list(args(d))
+    with pytest.raises(RuntimeError):
+        yamoe_amd.experts(a[0].view(2, 4, 64), *a[1:], 8, 4, 2)  # hidden must be 2D
+    with pytest.raises(RuntimeError):
+        yamoe_amd.experts(*a, 8, 5, 2)  # num_experts disagrees with the weights
+    with pytest.raises(RuntimeError):
+        yamoe_amd.experts(a[0], a[1], a[2].float(), *a[3:], 8, 4, 2)  # dtype mismatch
+    with pytest.raises(RuntimeError):
+        yamoe_amd.experts(a[0], a[1].float(), *a[2:], 8, 4, 2)  # indices must be integers

@@ -1,0 +1,101 @@
+"""Routing, permute and combine kernels against the oracle: integer results bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import yamoe_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # N, E, capacity, index dtype, with invalid ids
+    (1, 1, 1, torch.int64, False),
+    (256, 128, 64, torch.int64, False),      # decode shape
+    (16384, 32, 4096, torch.int64, False),   # GPT-OSS-20B shape
+    (8192, 8, 256, torch.int32, False),      # README shape with the literal README capacity
+    (1000, 7, 100, torch.int32, True),
+    (32768, 768, 40, torch.int64, True),     # largest single-block case, most buckets
+    (65536, 128, 16384, torch.int64, False),  # multi-block form
+    (40001, 5, 9000, torch.int32, True),
+    (0, 4, 3, torch.int64, False),
+]
+
+
+@pytest.mark.parametrize("N,E,C,dt,invalid", CASES)
+def test_route_bit_exact(gpu, N, E, C, dt, invalid):
+    from yamoe_amd import _cabi
+    print("route N=%d E=%d C=%d %s" % (N, E, C, dt), flush=True)
+    rng = np.random.default_rng(N + E)
+    # skewed popularity so that some experts are empty and some overflow the capacity
+    p = rng.random(E) ** 3
+    ids = rng.choice(E, size=N, p=p / p.sum()) if N else np.zeros(0, dtype=np.int64)
+    if invalid and N:
+        ids[rng.integers(0, N, size=N // 50 + 1)] = E + 3
+        ids[rng.integers(0, N, size=N // 50 + 1)] = -2
+    want = O.route(ids, E, C)
+    t = torch.from_numpy(ids.astype(np.int64)).to(dt).to(gpu)
+    se, si, counts, offsets, inv = _cabi.route(t, E, C)
+    torch.cuda.synchronize()
+    assert np.array_equal(counts.cpu().numpy(), want["counts"])
+    assert np.array_equal(offsets.cpu().numpy(), want["offsets"])
+    assert np.array_equal(si.cpu().numpy(), want["sorted_idx"])
+    assert np.array_equal(se.cpu().numpy(), want["sorted_expert"])
+    assert np.array_equal(inv.cpu().numpy(), want["inv_pos"])
+
+
+def test_route_zipf_config(gpu):
+    from yamoe_amd import _cabi
+    from yamoe_amd.workloads import make_config
+    d, c = make_config("zipf", weights=False)
+    idx = d["router_indices"]
+    want = O.route(idx.numpy(), c["E"], c["T"])
+    se, si, counts, offsets, inv = _cabi.route(idx.to(gpu), c["E"], c["T"])
+    assert np.array_equal(si.cpu().numpy(), want["sorted_idx"])
+    assert np.array_equal(counts.cpu().numpy(), want["counts"])
+    assert np.array_equal(inv.cpu().numpy(), want["inv_pos"])
+    assert (want["counts"] == 0).sum() > 0 and want["counts"].max() > 10 * want["counts"].mean()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,K,E,H", [(64, 4, 16, 2880), (300, 2, 5, 72), (7, 3, 4, 10)])
+def test_permute_and_combine(gpu, dtype, T, K, E, H):
+    from yamoe_amd import _cabi
+    print("permute/combine", dtype, T, K, E, H, flush=True)
+    g = torch.Generator().manual_seed(T + H)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    idx = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)])
+    C = max(1, (T * K) // (2 * E))  # some slots get dropped
+    r = O.route(idx.numpy(), E, C)
+    se, si, counts, offsets, inv = _cabi.route(idx.to(gpu), E, C)
+    xp = _cabi.permute(x.to(gpu), si, K)
+    want_xp = x[torch.from_numpy(r["sorted_idx"].astype(np.int64)) // K]
+    assert torch.equal(xp.cpu(), want_xp)  # a copy: bit-exact
+
+    # combine: rows of y_perm weighted by dense routing weights, dropped slots skipped
+    y = torch.randn(T * K, H, generator=g).to(dtype)
+    rw = torch.rand(T, E, generator=g).to(dtype)
+    got = _cabi.combine(y.to(gpu), inv, idx.to(gpu), rw.to(gpu), T, K, E).cpu()
+    want = torch.zeros(T, H, dtype=torch.float64)
+    invp = r["inv_pos"].reshape(T, K)
+    for t in range(T):
+        for k in range(K):
+            if invp[t, k] >= 0:
+                want[t] += rw[t, idx[t, k]].double() * y[invp[t, k]].double()
+    tol = 1e-6 if dtype == torch.float32 else 1e-2
+    assert O.rel_l2(got, want) < tol
+    # per-slot [T,K] weights give the same result as the dense layout
+    sel = torch.gather(rw, 1, idx)
+    got_k = _cabi.combine(y.to(gpu), inv, idx.to(gpu), sel.to(gpu), T, K, E).cpu()
+    assert torch.equal(got_k, got)
+    # weight 1 (the backward of the permute)
+    got1 = _cabi.combine(y.to(gpu), inv, None, None, T, K, E).cpu()
+    want1 = torch.zeros(T, H, dtype=torch.float64)
+    for t in range(T):
+        for k in range(K):
+            if invp[t, k] >= 0:
+                want1[t] += y[invp[t, k]].double()
+    assert O.rel_l2(got1, want1) < tol
+    # tokens whose slots were all dropped come out as exact zeros
+    all_dropped = (invp < 0).all(axis=1)
+    if all_dropped.any():
+        assert torch.all(got[torch.from_numpy(all_dropped)] == 0)

@@ -1,0 +1,226 @@
+"""Pins the CPU oracle (oracle/yamoe_oracle.py) against things that do not share its code:
+brute force, library routines, closed-form special cases, finite differences and a hand-made
+known-answer fixture.  The reference ships no fixtures for this path, so these are the anchors."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import yamoe_oracle as O
+from yamoe_amd.workloads import make_inputs
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+# ---- routing ---------------------------------------------------------------------------------------
+def brute_route(ids, E, C):
+    """O(N^2) definition: position = #(smaller keys) + #(equal keys at lower index)."""
+    N = len(ids)
+    key = [E if (v < 0 or v >= E) else v for v in ids]
+    pos = [sum(1 for j in range(N) if key[j] < key[i] or (key[j] == key[i] and j < i)) for i in range(N)]
+    sorted_idx = [0] * N
+    for i, p in enumerate(pos):
+        sorted_idx[p] = i
+    counts = [sum(1 for k in key if k == e) for e in range(E)]
+    inv = []
+    for i in range(N):
+        rank = sum(1 for j in range(i) if key[j] == key[i])
+        inv.append(pos[i] if key[i] < E and rank < C else -1)
+    return sorted_idx, counts, inv
+
+
+@pytest.mark.parametrize("N,E,C,seed", [(1, 1, 1, 0), (17, 3, 100, 1), (64, 8, 5, 2), (200, 130, 2, 3), (97, 5, 0, 4)])
+def test_route_matches_brute_force(N, E, C, seed):
+    rng = np.random.default_rng(seed)
+    ids = rng.integers(0, E, size=N)
+    if N > 10:
+        ids[3] = -1  # invalid ids sort last and are dropped
+        ids[7] = E + 2
+    r = O.route(ids, E, C)
+    sidx, counts, inv = brute_route(ids.tolist(), E, C)
+    assert r["sorted_idx"].tolist() == sidx
+    assert r["counts"].tolist() == counts
+    assert r["inv_pos"].tolist() == inv
+    assert r["offsets"].tolist() == [0] + np.cumsum(counts).tolist()
+    assert r["bins"].tolist() == np.cumsum(counts).tolist()
+    assert r["sorted_expert"].tolist() == ids[np.array(sidx, dtype=np.int64)].tolist() if N else True
+
+
+def test_route_invariants_large():
+    rng = np.random.default_rng(5)
+    ids = rng.integers(0, 128, size=65536)
+    r = O.route(ids, 128, 700)
+    assert sorted(r["sorted_idx"].tolist()) == list(range(65536))
+    se = r["sorted_expert"]
+    assert np.all(se[1:] >= se[:-1])
+    same = se[1:] == se[:-1]
+    assert np.all(r["sorted_idx"][1:][same] > r["sorted_idx"][:-1][same])  # stability
+    kept = r["inv_pos"] >= 0
+    assert kept.sum() == np.minimum(r["counts"], 700).sum()
+    assert np.all(r["sorted_idx"][r["inv_pos"][kept]] == np.nonzero(kept)[0])
+
+
+def test_route_empty():
+    r = O.route(np.zeros(0, dtype=np.int64), 4, 3)
+    assert r["counts"].tolist() == [0, 0, 0, 0] and r["offsets"].tolist() == [0] * 5
+
+
+# ---- GLU ---------------------------------------------------------------------------------------------
+def test_glu_known_answers():
+    with open(os.path.join(HERE, "golden", "glu_kat.json")) as f:
+        kat = json.load(f)
+    gu = torch.tensor([[c["G"], c["U"]] for c in kat], dtype=torch.float64)
+    got = O.glu(gu)[:, 0]
+    want = torch.tensor([c["h"] for c in kat], dtype=torch.float64)
+    assert torch.allclose(got, want, rtol=1e-12, atol=1e-15)
+
+
+def test_glu_uses_even_gate_odd_up():
+    gu = torch.tensor([[2.0, -1.0, 0.0, 5.0]], dtype=torch.float64)  # pairs (G=2,U=-1), (G=0,U=5)
+    assert O.glu(gu).tolist() == [[0.0, 0.0]]  # U=-1 kills the first, G=0 the second
+    gu = torch.tensor([[-1.0, 2.0]], dtype=torch.float64)  # swapped roles would give 0
+    assert O.glu(gu)[0, 0].item() != 0.0
+
+
+# ---- forward -------------------------------------------------------------------------------------------
+def tiny(seed=0, T=24, H=16, I=12, E=4, K=2, dtype=torch.float64, **kw):
+    d = make_inputs(T, H, I, E, K, torch.float32, seed=seed, w_std=0.3, bias_std=0.2, **kw)
+    return {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in d.items()}
+
+
+def args(d):
+    return (d["hidden"], d["router_indices"], d["routing_weights"], d["gate_up_proj"], d["gate_up_proj_bias"],
+            d["down_proj"], d["down_proj_bias"])
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_loop_equals_dense_formulation(seed):
+    d = tiny(seed)
+    a = O.experts_loop(*args(d))
+    b = O.experts_dense(d["hidden"], d["routing_weights"], d["gate_up_proj"], d["gate_up_proj_bias"],
+                        d["down_proj"], d["down_proj_bias"])
+    assert O.rel_l2(a, b) < 1e-13
+
+
+def test_single_expert_is_one_mlp():
+    d = tiny(2, E=1, K=1)
+    x = d["hidden"]
+    gu = x @ d["gate_up_proj"][0] + d["gate_up_proj_bias"][0]
+    G, U = gu[:, 0::2], gu[:, 1::2]
+    h = (U.clamp(-7, 7) + 1) * torch.minimum(G, torch.tensor(7.0, dtype=G.dtype)) * \
+        torch.sigmoid(1.702 * torch.minimum(G, torch.tensor(7.0, dtype=G.dtype)))
+    want = (h @ d["down_proj"][0] + d["down_proj_bias"][0]) * d["routing_weights"][:, :1]
+    assert O.rel_l2(O.experts_loop(*args(d)), want) < 1e-13
+
+
+def test_zero_weights_reduce_to_bias_closed_form():
+    d = tiny(3)
+    d["gate_up_proj"].zero_()
+    out = O.experts_loop(*args(d))
+    # every token of expert e gets the same vector f(bgu[e]) @ Wd[e] + bd[e]
+    E = d["gate_up_proj"].shape[0]
+    per_e = torch.stack([O.glu(d["gate_up_proj_bias"][e][None])[0] @ d["down_proj"][e] + d["down_proj_bias"][e]
+                         for e in range(E)])
+    want = d["routing_weights"] @ per_e
+    assert O.rel_l2(out, want) < 1e-13
+
+
+def test_interleaved_identity_weights_copy_rows():
+    # Wgu[e][:, 2j] = Wgu[e][:, 2j+1] = unit vector j  =>  G = U = x, so act = glu applied to (x, x)
+    d = tiny(4, H=8, I=8)
+    E, H, _ = d["gate_up_proj"].shape
+    w = torch.zeros_like(d["gate_up_proj"])
+    for j in range(H):
+        w[:, j, 2 * j] = 1
+        w[:, j, 2 * j + 1] = 1
+    d["gate_up_proj"], d["gate_up_proj_bias"] = w, torch.zeros_like(d["gate_up_proj_bias"])
+    d["down_proj"] = torch.eye(H, dtype=w.dtype).repeat(E, 1, 1)
+    d["down_proj_bias"].zero_()
+    x = d["hidden"]
+    g = x.clamp(max=7)
+    act = (x.clamp(-7, 7) + 1) * g * torch.sigmoid(1.702 * g)
+    want = act * d["routing_weights"].sum(1, keepdim=True)
+    assert O.rel_l2(O.experts_loop(*args(d)), want) < 1e-13
+
+
+def test_linear_in_routing_weights():
+    d = tiny(5)
+    a = O.experts_loop(*args(d))
+    d2 = dict(d)
+    d2["routing_weights"] = d["routing_weights"] * 3.0
+    assert O.rel_l2(O.experts_loop(*args(d2)), 3.0 * a) < 1e-13
+
+
+def brute_capacity(d, C):
+    """Per-slot loops following binned_gather / binned_scatter (yamoe_ref.py:4-35)."""
+    x, idx, rw = d["hidden"], d["router_indices"], d["routing_weights"]
+    T, K = idx.shape
+    E = rw.shape[1]
+    out = torch.zeros_like(x)
+    seen = [0] * E
+    order = sorted(range(T * K), key=lambda f: (int(idx.view(-1)[f]), f))
+    for f in order:
+        e = int(idx.view(-1)[f])
+        if seen[e] >= C:
+            continue
+        seen[e] += 1
+        t = f // K
+        gu = x[t] @ d["gate_up_proj"][e] + d["gate_up_proj_bias"][e]
+        y = O.glu(gu[None])[0] @ d["down_proj"][e] + d["down_proj_bias"][e]
+        out[t] += y * rw[t, e]
+    return out
+
+
+@pytest.mark.parametrize("C", [0, 1, 5, 1000])
+def test_capacity_matches_brute_force(C):
+    d = tiny(6)
+    got = O.experts_capacity(*args(d), C)
+    want = brute_capacity(d, C)
+    assert O.max_abs(got, want) < 1e-12
+
+
+def test_capacity_large_equals_loop_and_slot_weights():
+    d = tiny(7)
+    a = O.experts_capacity(*args(d), 10 ** 6)
+    assert O.rel_l2(a, O.experts_loop(*args(d))) < 1e-13
+    sel = torch.gather(d["routing_weights"], 1, d["router_indices"])  # [T,K] layout gives the same result
+    b = O.experts_capacity(d["hidden"], d["router_indices"], sel, d["gate_up_proj"], d["gate_up_proj_bias"],
+                           d["down_proj"], d["down_proj_bias"], 10 ** 6)
+    assert O.rel_l2(b, a) < 1e-13
+
+
+# ---- backward ------------------------------------------------------------------------------------------
+def test_backward_gradcheck_fp64():
+    d = tiny(8, T=6, H=8, I=4, E=3, K=2)
+    idx = d["router_indices"]
+    leaves = [d[k].clone().requires_grad_(True) for k in
+              ("hidden", "routing_weights", "gate_up_proj", "gate_up_proj_bias", "down_proj", "down_proj_bias")]
+
+    def f(h, rw, wgu, bgu, wd, bd):
+        return O.experts_capacity(h, idx, rw, wgu, bgu, wd, bd, 3)
+
+    assert torch.autograd.gradcheck(f, leaves, eps=1e-6, atol=1e-6, rtol=1e-4)
+
+
+@pytest.mark.parametrize("C,slot_weights", [(1000, False), (4, False), (1000, True)])
+def test_backward_closed_form_equals_autograd(C, slot_weights):
+    d = tiny(9)
+    if slot_weights:
+        d["routing_weights"] = torch.gather(d["routing_weights"], 1, d["router_indices"])
+    gy = torch.randn(d["hidden"].shape, dtype=torch.float64, generator=torch.Generator().manual_seed(1))
+    a = O.experts_backward(gy, *args(d), C, compute_dtype=torch.float64)
+    b = O.experts_backward_closed(gy, *args(d), C)
+    for ga, gb in zip(a, b):
+        assert ga.shape == gb.shape
+        assert O.max_abs(ga, gb) < 1e-10
+
+
+def test_backward_routing_grad_is_zero_outside_selection():
+    d = tiny(10)
+    gy = torch.ones_like(d["hidden"])
+    d_rw = O.experts_backward(gy, *args(d), 1000, compute_dtype=torch.float64)[1]
+    sel = torch.zeros_like(d_rw, dtype=torch.bool).scatter_(1, d["router_indices"], True)
+    assert torch.all(d_rw[~sel] == 0)
+    assert torch.any(d_rw[sel] != 0)

@@ -1,0 +1,350 @@
+// C ABI of libyamoe_hip.so: argument checks, workspace carving and the launch sequences of the
+// forward (csrc/moe.cpp:45-223) and backward (csrc/experts_backward.cu:126-341) expert layer.
+// No allocation, no host synchronisation, every launch on the caller's stream.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "common.h"
+
+namespace yamoe {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+int check_launch(const char *what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("%s: %s", what, hipGetErrorString(e));
+    return (int)e;
+  }
+  return 0;
+}
+
+// kernels defined in the other translation units
+template <typename T> int launch_permute(const void *, const int *, void *, int, int, int, hipStream_t);
+template <typename T>
+int launch_combine(const void *, const int *, const void *, int, const void *, int, void *, int, int, int, int,
+                   hipStream_t);
+template <typename T>
+int launch_combine_backward(const void *, const void *, const int *, const int *, const void *, int, const void *,
+                            int, void *, void *, int, int, int, int, hipStream_t);
+template <typename T>
+int launch_expert_colsum(const void *, const int *, const int *, int, void *, int, int, hipStream_t);
+template <typename T>
+int gemm_gate_up(const void *, const int *, const void *, const void *, void *, void *, const void *, int, int, int,
+                 int, int, hipStream_t);
+template <typename T>
+int gemm_down(const void *, const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);
+template <typename T>
+int gemm_dgrad(const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);
+template <typename T>
+int gemm_wgrad(const void *, const void *, void *, const int *, const int *, int, int, int, int, hipStream_t);
+template <typename T> int glu_backward_rows(const void *, const void *, void *, long long, hipStream_t);
+template <typename T>
+int stream_gate_up(const void *, const int *, const void *, const void *, void *, void *, const void *, int, int, int,
+                   int, int, hipStream_t);
+template <typename T>
+int stream_down(const void *, const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);
+
+template <typename T> struct HasStreamPath { static constexpr bool value = sizeof(T) == 2; };
+
+__global__ void fill_zero_kernel(uint32_t *p, long long n_words) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  long long stride = (long long)gridDim.x * blockDim.x;
+  for (; i < n_words; i += stride) p[i] = 0u;
+}
+static int fill_zero(void *p, size_t bytes, hipStream_t stream) {
+  long long words = (long long)((bytes + 3) / 4);
+  if (words == 0) return 0;
+  long long blocks = (words + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (uint32_t *)p, words);
+  return check_launch("fill_zero_kernel");
+}
+
+static int check_problem(const yamoe_problem *p, const char *who) {
+  if (!p) { set_error("%s: null problem", who); return YAMOE_E_ARG; }
+  if (p->T < 0 || p->K <= 0 || p->E <= 0 || p->H <= 0 || p->I <= 0) {
+    set_error("%s: need T >= 0 and K, E, H, I > 0 (T=%d K=%d E=%d H=%d I=%d)", who, p->T, p->K, p->E, p->H, p->I);
+    return YAMOE_E_ARG;
+  }
+  if (p->dtype != YAMOE_F32 && p->dtype != YAMOE_F16 && p->dtype != YAMOE_BF16) {
+    set_error("%s: unknown dtype %d", who, p->dtype);
+    return YAMOE_E_DTYPE;
+  }
+  int vec = 16 / (int)dtype_size(p->dtype);
+  if (p->H % vec != 0 || p->I % vec != 0) {
+    set_error("%s: H and I must be multiples of %d for this dtype (H=%d I=%d)", who, vec, p->H, p->I);
+    return YAMOE_E_ARG;
+  }
+  if (p->rw_cols != p->E && p->rw_cols != p->K) {
+    set_error("%s: routing_weights must be [T,E] or [T,K] (got %d columns, E=%d K=%d)", who, p->rw_cols, p->E, p->K);
+    return YAMOE_E_ARG;
+  }
+  if ((long long)p->T * p->K > 0x7fffffffLL / 2) {
+    set_error("%s: T*K too large", who);
+    return YAMOE_E_ARG;
+  }
+  return 0;
+}
+
+// Carves 256-byte aligned regions out of the workspace.
+struct Carver {
+  char *base;
+  size_t used = 0;
+  explicit Carver(void *b) : base((char *)b) {}
+  void *take(size_t bytes) {
+    void *p = base ? base + used : nullptr;
+    used += align_up(bytes == 0 ? 1 : bytes, 256);
+    return p;
+  }
+};
+
+struct ForwardBuffers {
+  int *sorted_expert, *sorted_idx, *inv_pos, *counts, *offsets;
+  void *schedule, *route_ws, *act, *y_perm;
+  size_t schedule_bytes, route_ws_bytes;
+};
+
+static size_t carve_forward(const yamoe_problem *p, void *ws, ForwardBuffers *b) {
+  const size_t N = (size_t)p->T * p->K, es = dtype_size(p->dtype);
+  Carver c(ws);
+  b->sorted_expert = (int *)c.take(N * 4);
+  b->sorted_idx = (int *)c.take(N * 4);
+  b->inv_pos = (int *)c.take(N * 4);
+  b->counts = (int *)c.take((size_t)p->E * 4);
+  b->offsets = (int *)c.take(((size_t)p->E + 1) * 4);
+  b->schedule_bytes = yamoe_schedule_bytes((int)N, p->E);
+  b->schedule = c.take(b->schedule_bytes);
+  b->route_ws_bytes = yamoe_route_workspace_bytes((int)N, p->E);
+  b->route_ws = c.take(b->route_ws_bytes);
+  b->act = c.take(N * p->I * es);
+  b->y_perm = c.take(N * p->H * es);
+  return c.used;
+}
+
+struct BackwardBuffers {
+  ForwardBuffers f;
+  void *x_perm, *pre, *g_y_perm, *d_act, *d_pre, *d_x_perm;
+};
+
+static size_t carve_backward(const yamoe_problem *p, void *ws, BackwardBuffers *b) {
+  size_t used = carve_forward(p, ws, &b->f);
+  const size_t N = (size_t)p->T * p->K, es = dtype_size(p->dtype);
+  Carver c(ws ? (char *)ws + used : nullptr);
+  b->x_perm = c.take(N * p->H * es);
+  b->pre = c.take(N * 2 * p->I * es);
+  b->g_y_perm = c.take(N * p->H * es);
+  b->d_pre = c.take(N * 2 * p->I * es);
+  // d_act reuses y_perm (dead after the combine backward); d_x_perm reuses g_y_perm's successor slot
+  b->d_act = b->f.y_perm;
+  b->d_x_perm = c.take(N * p->H * es);
+  return used + c.used;
+}
+
+#define YAMOE_TRY(expr)        \
+  do {                         \
+    int rc_ = (expr);          \
+    if (rc_ != 0) return rc_;  \
+  } while (0)
+
+template <typename T>
+static int forward_impl(const yamoe_problem *p, const void *x, const void *idx, const void *rw, const void *wgu,
+                        const void *bgu, const void *wd, const void *bd, void *out, void *ws, hipStream_t stream) {
+  ForwardBuffers b;
+  carve_forward(p, ws, &b);
+  const int N = p->T * p->K;
+  void *st = (void *)stream;
+  if (N == 0 || p->T == 0) return 0;
+  YAMOE_TRY(yamoe_route(idx, p->idx_i64, N, p->E, p->capacity, b.sorted_expert, b.sorted_idx, b.counts, b.offsets,
+                        b.inv_pos, b.route_ws, b.route_ws_bytes, st));
+  const int stream_rows = HasStreamPath<T>::value ? kStreamMaxRows : 0;
+  YAMOE_TRY(yamoe_build_schedule(b.counts, b.offsets, N, p->E, p->capacity, stream_rows, b.schedule, b.schedule_bytes,
+                                 st));
+  YAMOE_TRY(gemm_gate_up<T>(x, b.sorted_idx, wgu, bgu, b.act, nullptr, b.schedule, N, p->K, p->E, p->H, p->I, stream));
+  if constexpr (HasStreamPath<T>::value)
+    YAMOE_TRY(stream_gate_up<T>(x, b.sorted_idx, wgu, bgu, b.act, nullptr, b.schedule, N, p->K, p->E, p->H, p->I,
+                                stream));
+  YAMOE_TRY(gemm_down<T>(b.act, wd, bd, b.y_perm, b.schedule, N, p->E, p->H, p->I, stream));
+  if constexpr (HasStreamPath<T>::value)
+    YAMOE_TRY(stream_down<T>(b.act, wd, bd, b.y_perm, b.schedule, N, p->E, p->H, p->I, stream));
+  YAMOE_TRY(launch_combine<T>(b.y_perm, b.inv_pos, idx, p->idx_i64, rw, p->rw_cols, out, p->T, p->K, p->E, p->H,
+                              stream));
+  return 0;
+}
+
+template <typename T>
+static int backward_impl(const yamoe_problem *p, const void *gy, const void *x, const void *idx, const void *rw,
+                         const void *wgu, const void *bgu, const void *wd, const void *bd, void *d_x, void *d_rw,
+                         void *d_wgu, void *d_bgu, void *d_wd, void *d_bd, void *ws, hipStream_t stream) {
+  BackwardBuffers b;
+  carve_backward(p, ws, &b);
+  const int N = p->T * p->K, E = p->E, H = p->H, I = p->I, cap = p->capacity < 0 ? 0 : p->capacity;
+  const size_t es = sizeof(T);
+  void *st = (void *)stream;
+  YAMOE_TRY(fill_zero(d_rw, (size_t)p->T * p->rw_cols * es, stream));
+  if (N == 0) {
+    YAMOE_TRY(fill_zero(d_wgu, (size_t)E * H * 2 * I * es, stream));
+    YAMOE_TRY(fill_zero(d_bgu, (size_t)E * 2 * I * es, stream));
+    YAMOE_TRY(fill_zero(d_wd, (size_t)E * I * H * es, stream));
+    YAMOE_TRY(fill_zero(d_bd, (size_t)E * H * es, stream));
+    return 0;
+  }
+  YAMOE_TRY(yamoe_route(idx, p->idx_i64, N, E, cap, b.f.sorted_expert, b.f.sorted_idx, b.f.counts, b.f.offsets,
+                        b.f.inv_pos, b.f.route_ws, b.f.route_ws_bytes, st));
+  YAMOE_TRY(yamoe_build_schedule(b.f.counts, b.f.offsets, N, E, cap, 0, b.f.schedule, b.f.schedule_bytes, st));
+  // forward recompute, keeping the pre-activations
+  YAMOE_TRY(launch_permute<T>(x, b.f.sorted_idx, b.x_perm, N, p->K, H, stream));
+  YAMOE_TRY(gemm_gate_up<T>(x, b.f.sorted_idx, wgu, bgu, b.f.act, b.pre, b.f.schedule, N, p->K, E, H, I, stream));
+  YAMOE_TRY(gemm_down<T>(b.f.act, wd, bd, b.f.y_perm, b.f.schedule, N, E, H, I, stream));
+  // combine backward: g_y_perm = grad_out[tok] * w, d_routing = <grad_out[tok], y_perm>
+  YAMOE_TRY(launch_combine_backward<T>(gy, b.f.y_perm, b.f.sorted_idx, b.f.inv_pos, idx, p->idx_i64, rw, p->rw_cols,
+                                       b.g_y_perm, d_rw, N, p->K, E, H, stream));
+  // down projection
+  YAMOE_TRY(launch_expert_colsum<T>(b.g_y_perm, b.f.counts, b.f.offsets, cap, d_bd, E, H, stream));
+  YAMOE_TRY(gemm_dgrad<T>(b.g_y_perm, wd, b.d_act, b.f.schedule, N, E, /*Kd=*/H, /*Nd=*/I, stream));
+  YAMOE_TRY(gemm_wgrad<T>(b.f.act, b.g_y_perm, d_wd, b.f.counts, b.f.offsets, cap, E, /*Md=*/I, /*Nd=*/H, stream));
+  // GLU
+  YAMOE_TRY(glu_backward_rows<T>(b.d_act, b.pre, b.d_pre, (long long)N * I, stream));
+  // gate_up projection
+  YAMOE_TRY(launch_expert_colsum<T>(b.d_pre, b.f.counts, b.f.offsets, cap, d_bgu, E, 2 * I, stream));
+  YAMOE_TRY(gemm_dgrad<T>(b.d_pre, wgu, b.d_x_perm, b.f.schedule, N, E, /*Kd=*/2 * I, /*Nd=*/H, stream));
+  YAMOE_TRY(gemm_wgrad<T>(b.x_perm, b.d_pre, d_wgu, b.f.counts, b.f.offsets, cap, E, /*Md=*/H, /*Nd=*/2 * I, stream));
+  // permute backward: d_hidden[t] = sum_k d_x_perm[inv_pos[t,k]]
+  YAMOE_TRY(launch_combine<T>(b.d_x_perm, b.f.inv_pos, idx, p->idx_i64, nullptr, p->K, d_x, p->T, p->K, E, H, stream));
+  return 0;
+}
+
+}  // namespace yamoe
+
+using namespace yamoe;
+
+#define YAMOE_DISPATCH(dtype, CALL)                                       \
+  switch (dtype) {                                                        \
+    case YAMOE_F32: { typedef float T; return CALL; }                     \
+    case YAMOE_BF16: { typedef bf16_t T; return CALL; }                   \
+    case YAMOE_F16: { typedef f16_t T; return CALL; }                     \
+    default: set_error("unknown dtype %d", dtype); return YAMOE_E_DTYPE;  \
+  }
+
+extern "C" int yamoe_abi_version(void) { return YAMOE_ABI_VERSION; }
+extern "C" const char *yamoe_last_error(void) { return g_error; }
+
+static int check_gemm_shape(const char *who, int N, int E, int H, int I, int dtype) {
+  if (N < 0 || E <= 0 || H <= 0 || I <= 0) { set_error("%s: bad size", who); return YAMOE_E_ARG; }
+  if (dtype != YAMOE_F32 && dtype != YAMOE_F16 && dtype != YAMOE_BF16) {
+    set_error("%s: unknown dtype %d", who, dtype);
+    return YAMOE_E_DTYPE;
+  }
+  int vec = 16 / (int)dtype_size(dtype);
+  if (H % vec != 0 || I % vec != 0) {
+    set_error("%s: H and I must be multiples of %d for this dtype (H=%d I=%d)", who, vec, H, I);
+    return YAMOE_E_ARG;
+  }
+  return 0;
+}
+
+template <typename T>
+static int gate_up_both(const void *x, const int *sorted_idx, const void *w, const void *bias, void *act, void *pre,
+                        const void *sched, int N, int K, int E, int H, int I, hipStream_t stream) {
+  YAMOE_TRY(gemm_gate_up<T>(x, sorted_idx, w, bias, act, pre, sched, N, K, E, H, I, stream));
+  if constexpr (HasStreamPath<T>::value)
+    YAMOE_TRY(stream_gate_up<T>(x, sorted_idx, w, bias, act, pre, sched, N, K, E, H, I, stream));
+  return 0;
+}
+template <typename T>
+static int down_both(const void *act, const void *w, const void *bias, void *y, const void *sched, int N, int E, int H,
+                     int I, hipStream_t stream) {
+  YAMOE_TRY(gemm_down<T>(act, w, bias, y, sched, N, E, H, I, stream));
+  if constexpr (HasStreamPath<T>::value) YAMOE_TRY(stream_down<T>(act, w, bias, y, sched, N, E, H, I, stream));
+  return 0;
+}
+
+extern "C" int yamoe_gate_up(const void *x, const int32_t *sorted_idx, const void *gate_up_proj,
+                             const void *gate_up_proj_bias, void *act, void *pre_act, const void *schedule, int32_t N,
+                             int32_t K, int32_t E, int32_t H, int32_t I, int32_t dtype, void *stream) {
+  YAMOE_TRY(check_gemm_shape("yamoe_gate_up", N, E, H, I, dtype));
+  if (N == 0) return 0;
+  if (!x || !sorted_idx || !gate_up_proj || !act || !schedule || K <= 0) {
+    set_error("yamoe_gate_up: null pointer or K <= 0");
+    return YAMOE_E_ARG;
+  }
+  YAMOE_DISPATCH(dtype, gate_up_both<T>(x, sorted_idx, gate_up_proj, gate_up_proj_bias, act, pre_act, schedule, N, K,
+                                        E, H, I, (hipStream_t)stream));
+}
+
+extern "C" int yamoe_down(const void *act, const void *down_proj, const void *down_proj_bias, void *y_perm,
+                          const void *schedule, int32_t N, int32_t E, int32_t H, int32_t I, int32_t dtype,
+                          void *stream) {
+  YAMOE_TRY(check_gemm_shape("yamoe_down", N, E, H, I, dtype));
+  if (N == 0) return 0;
+  if (!act || !down_proj || !y_perm || !schedule) {
+    set_error("yamoe_down: null pointer");
+    return YAMOE_E_ARG;
+  }
+  YAMOE_DISPATCH(dtype, down_both<T>(act, down_proj, down_proj_bias, y_perm, schedule, N, E, H, I,
+                                     (hipStream_t)stream));
+}
+
+extern "C" size_t yamoe_experts_workspace_bytes(const yamoe_problem *p) {
+  if (check_problem(p, "yamoe_experts_workspace_bytes")) return 0;
+  ForwardBuffers b;
+  return carve_forward(p, nullptr, &b);
+}
+
+extern "C" int yamoe_experts_forward(const yamoe_problem *p, const void *hidden_states, const void *router_indices,
+                                     const void *routing_weights, const void *gate_up_proj,
+                                     const void *gate_up_proj_bias, const void *down_proj, const void *down_proj_bias,
+                                     void *out, void *workspace, size_t workspace_bytes, void *stream) {
+  YAMOE_TRY(check_problem(p, "yamoe_experts_forward"));
+  if (p->T == 0) return 0;
+  if (!hidden_states || !router_indices || !routing_weights || !gate_up_proj || !gate_up_proj_bias || !down_proj ||
+      !down_proj_bias || !out || !workspace) {
+    set_error("yamoe_experts_forward: null pointer");
+    return YAMOE_E_ARG;
+  }
+  size_t need = yamoe_experts_workspace_bytes(p);
+  if (workspace_bytes < need) {
+    set_error("yamoe_experts_forward: workspace too small (%zu < %zu)", workspace_bytes, need);
+    return YAMOE_E_WORKSPACE;
+  }
+  YAMOE_DISPATCH(p->dtype, forward_impl<T>(p, hidden_states, router_indices, routing_weights, gate_up_proj,
+                                           gate_up_proj_bias, down_proj, down_proj_bias, out, workspace,
+                                           (hipStream_t)stream));
+}
+
+extern "C" size_t yamoe_experts_backward_workspace_bytes(const yamoe_problem *p) {
+  if (check_problem(p, "yamoe_experts_backward_workspace_bytes")) return 0;
+  BackwardBuffers b;
+  return carve_backward(p, nullptr, &b);
+}
+
+extern "C" int yamoe_experts_backward(const yamoe_problem *p, const void *grad_out, const void *hidden_states,
+                                      const void *router_indices, const void *routing_weights,
+                                      const void *gate_up_proj, const void *gate_up_proj_bias, const void *down_proj,
+                                      const void *down_proj_bias, void *d_hidden, void *d_routing,
+                                      void *d_gate_up_proj, void *d_gate_up_proj_bias, void *d_down_proj,
+                                      void *d_down_proj_bias, void *workspace, size_t workspace_bytes, void *stream) {
+  YAMOE_TRY(check_problem(p, "yamoe_experts_backward"));
+  if (!gate_up_proj || !gate_up_proj_bias || !down_proj || !down_proj_bias || !d_gate_up_proj ||
+      !d_gate_up_proj_bias || !d_down_proj || !d_down_proj_bias || !workspace ||
+      (p->T > 0 && (!grad_out || !hidden_states || !router_indices || !routing_weights || !d_hidden || !d_routing))) {
+    set_error("yamoe_experts_backward: null pointer");
+    return YAMOE_E_ARG;
+  }
+  size_t need = yamoe_experts_backward_workspace_bytes(p);
+  if (workspace_bytes < need) {
+    set_error("yamoe_experts_backward: workspace too small (%zu < %zu)", workspace_bytes, need);
+    return YAMOE_E_WORKSPACE;
+  }
+  YAMOE_DISPATCH(p->dtype, backward_impl<T>(p, grad_out, hidden_states, router_indices, routing_weights, gate_up_proj,
+                                            gate_up_proj_bias, down_proj, down_proj_bias, d_hidden, d_routing,
+                                            d_gate_up_proj, d_gate_up_proj_bias, d_down_proj, d_down_proj_bias,
+                                            workspace, (hipStream_t)stream));
+}

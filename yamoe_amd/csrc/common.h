@@ -1,0 +1,110 @@
+// Shared device/host helpers for the gfx950 expert-layer kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/yamoe_hip.h"
+
+namespace yamoe {
+
+constexpr int kWave = 64;
+
+// Clamped-SwiGLU constants of the GPT-OSS expert MLP (csrc/moe.cpp:175-179).
+constexpr float kGluLimit = 7.0f;
+constexpr float kGluAlpha = 1.702f;
+
+// Experts with at most this many kept rows take the weight-streaming path.
+constexpr int kStreamMaxRows = 16;
+
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <typename T> struct ElemTraits;
+template <> struct ElemTraits<float> {
+  static constexpr int kDtype = YAMOE_F32;
+  static constexpr int kVec = 4;  // elements per 16-byte chunk
+  __device__ static inline float to_f32(float v) { return v; }
+  __device__ static inline float from_f32(float v) { return v; }
+};
+template <> struct ElemTraits<bf16_t> {
+  static constexpr int kDtype = YAMOE_BF16;
+  static constexpr int kVec = 8;
+  __device__ static inline float to_f32(bf16_t v) { return (float)v; }
+  __device__ static inline bf16_t from_f32(float v) { return (bf16_t)v; }
+};
+template <> struct ElemTraits<f16_t> {
+  static constexpr int kDtype = YAMOE_F16;
+  static constexpr int kVec = 8;
+  __device__ static inline float to_f32(f16_t v) { return (float)v; }
+  __device__ static inline f16_t from_f32(float v) { return (f16_t)v; }
+};
+
+__host__ __device__ inline size_t dtype_size(int dtype) { return dtype == YAMOE_F32 ? 4 : 2; }
+
+__host__ __device__ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+__host__ __device__ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// h = (clamp(U,-L,L) + 1) * g * sigmoid(alpha * g),  g = min(G, L)     (csrc/moe.cpp:164-180)
+__device__ inline float glu_forward(float G, float U) {
+  float g = fminf(G, kGluLimit);
+  float u = fminf(fmaxf(U, -kGluLimit), kGluLimit);
+  float s = 1.0f / (1.0f + __expf(-kGluAlpha * g));
+  return (u + 1.0f) * (g * s);
+}
+
+// Gradients of glu_forward with respect to G and U given dh (csrc/experts_backward.cu:285-299).
+__device__ inline void glu_backward(float G, float U, float dh, float &dG, float &dU) {
+  float g = fminf(G, kGluLimit);
+  float u = fminf(fmaxf(U, -kGluLimit), kGluLimit);
+  float s = 1.0f / (1.0f + __expf(-kGluAlpha * g));
+  float a = g * s;
+  dU = (U > kGluLimit || U < -kGluLimit) ? 0.0f : dh * a;
+  float dgl = dh * (u + 1.0f);
+  dG = (G > kGluLimit) ? 0.0f : dgl * (s + g * s * (1.0f - s) * kGluAlpha);
+}
+
+// ---- schedule: device-built work lists shared by the expert GEMM kernels ---------------------
+// Layout of the schedule region (int32 words):
+//   [0] n_row_tiles   number of (expert, row-block) entries for the MFMA kernels
+//   [1] n_small       number of experts on the weight-streaming path
+//   [2] n_active      experts with at least one kept row
+//   [3] n_kept        total kept rows
+//   [8 ...)           row tiles: 8 words each  {expert, first sorted row, valid rows,
+//                       index of the expert's first row tile, number of row tiles of the expert, 0,0,0}
+//   then              small experts: 4 words each {expert, first sorted row, valid rows, 0}
+constexpr int kRowTile = 256;  // rows of one MFMA row tile
+constexpr int kSchedHeader = 8;
+
+__host__ __device__ inline int sched_max_row_tiles(int N, int E) {
+  // every expert with kept rows adds at most one partly filled tile
+  return N / kRowTile + (N < E ? N : E) + 1;
+}
+__host__ __device__ inline int sched_max_small(int N, int E) { return (N < E ? N : E) + 1; }
+
+struct ScheduleView {
+  const int *hdr;
+  const int *row_tiles;
+  const int *small;
+};
+__host__ __device__ inline ScheduleView schedule_view(const void *p, int N, int E) {
+  const int *w = (const int *)p;
+  ScheduleView v;
+  v.hdr = w;
+  v.row_tiles = w + kSchedHeader;
+  v.small = w + kSchedHeader + 8 * sched_max_row_tiles(N, E);
+  return v;
+}
+
+// error reporting for the C ABI
+void set_error(const char *fmt, ...);
+int check_launch(const char *what);
+
+}  // namespace yamoe

@@ -1,0 +1,527 @@
+// Grouped expert GEMMs on gfx950 matrix cores.
+//
+// One workgroup (4 wavefronts, 2x2) computes a 256x256 output tile with 32x32 MFMA blocks
+// (v_mfma_f32_32x32x16_{bf16,f16}, v_mfma_f32_32x32x2_f32), fp32 accumulators, and walks the
+// contraction in slabs of 128 bytes per row (64 half-precision or 32 fp32 values).  Both operands
+// sit in LDS as [row][k] with k contiguous, so a lane's MFMA operand is one 16-byte ds_read.
+//
+//  * An operand that is k-contiguous in memory (activations, or weights read "transposed" in the
+//    data-gradient products) is copied slab by slab: 8 consecutive lanes fetch the 128 bytes of
+//    one row.
+//  * An operand that is contiguous along the other axis (the forward weights [K,N], and both
+//    operands of the weight-gradient products) is fetched as 16-byte pieces of V consecutive
+//    columns for V consecutive k (V = 8 halves or 4 floats), transposed in registers (v_perm_b32
+//    for 16-bit data, pure renaming for fp32) and written as V 16-byte k-runs.  8 consecutive lanes
+//    hold the 8 k-blocks of one column group, so each LDS write instruction fills whole rows.
+//
+// The 16-byte chunks of an LDS row are XOR-swizzled with the row number so that the MFMA operand
+// reads (32 consecutive rows, same chunk) spread over all banks.
+//
+// Global loads of slab s+1 are issued before the MFMAs of slab s and written to the other LDS
+// buffer afterwards: one barrier per slab.
+//
+// Tile order: workgroup ids are dealt round-robin over the 8 XCDs by the hardware, so id b is
+// remapped to logical tile (b % 8) * per_xcd + b / 8.  Logical tiles run expert-major, then
+// column tile, then the expert's row tiles, so the ~32 tiles in flight on one XCD share one
+// expert's weight column tiles and activation row tiles through that XCD's L2.
+//
+// Replaces batch_mm / torch::bmm on padded [E,C,*] buffers (csrc/batch_mm.cu:7-31) and the ATen
+// bias + clamped-SwiGLU chain (csrc/moe.cpp:161-187; backward csrc/experts_backward.cu:277-311).
+#include "common.h"
+
+namespace yamoe {
+
+constexpr int kBM = 256, kBN = 256;
+constexpr int kGemmThreads = 256;
+constexpr int kRowBytes = 128;                 // bytes of one LDS tile row (one K slab)
+constexpr int kTileBytes = kBM * kRowBytes;    // 32 KB per operand per stage
+constexpr int kGemmLds = 4 * kTileBytes;       // A,B x 2 stages = 128 KB
+constexpr int kXcds = 8;
+
+static_assert(kBM == kRowTile, "row tiles of the schedule must match the GEMM tile");
+
+enum { OP_KCONTIG = 0, OP_TRANSPOSED = 1 };
+enum {
+  EPI_STORE = 0,  // C = acc (+ bias)
+  EPI_GLU = 1     // act = glu(acc + bias) on interleaved gate/up columns (+ optional pre-activations)
+};
+enum { PROB_ROWS = 0, PROB_WGRAD = 1 };
+
+struct GemmArgs {
+  const void *A;         // PROB_ROWS: [rows, lda] k-contiguous.  PROB_WGRAD: [rows(k), lda] m-contiguous
+  const void *B;         // weights of all experts, or [rows(k), ldb] for PROB_WGRAD
+  const void *bias;      // [E, Nd] or null
+  void *C;               // output
+  void *C2;              // EPI_GLU: optional pre-activations [rows, Nd]
+  const int *a_rows;     // optional gather of A rows: source row = a_rows[p] / a_div
+  const int *sched;      // PROB_ROWS: schedule region
+  const int *counts;     // PROB_WGRAD: per-expert counts / offsets
+  const int *offsets;
+  int a_div;
+  int Kd, Nd, Md;        // contraction length, output columns; Md = output rows per expert (PROB_WGRAD)
+  int lda, ldb, ldc;     // leading dimensions in elements
+  long long b_expert_stride;  // elements between experts in B (PROB_ROWS)
+  long long c_expert_stride;  // elements between experts in C (PROB_WGRAD)
+  int n_col_tiles, n_row_tiles_wgrad;
+  int N, E, capacity;
+};
+
+__device__ inline int lds_swizzle(int row) { return (row ^ (row >> 3)) & 7; }
+__device__ inline int lds_chunk_off(int row, int chunk) {
+  return row * kRowBytes + ((chunk ^ lds_swizzle(row)) << 4);
+}
+
+template <typename T> struct Mma;
+template <> struct Mma<bf16_t> {
+  __device__ static inline void run(const u32x4 &a, const u32x4 &b, f32x16 &c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma<f16_t> {
+  __device__ static inline void run(const u32x4 &a, const u32x4 &b, f32x16 &c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                               __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma<float> {
+  __device__ static inline void run(const u32x4 &a, const u32x4 &b, f32x16 &c) {
+    const f32x4 af = __builtin_bit_cast(f32x4, a), bf = __builtin_bit_cast(f32x4, b);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) c = __builtin_amdgcn_mfma_f32_32x32x2f32(af[q], bf[q], c, 0, 0, 0);
+  }
+};
+
+// Transpose a VxV block held as V rows of 16 bytes into V columns of 16 bytes.
+template <int ESIZE> struct BlockTranspose;
+template <> struct BlockTranspose<2> {
+  __device__ static inline void run(const u32x4 (&r)[8], u32x4 (&c)[8]) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+        c[j][d] = __builtin_amdgcn_perm(r[2 * d + 1][j >> 1], r[2 * d][j >> 1], sel);
+    }
+  }
+};
+template <> struct BlockTranspose<4> {
+  // two independent 4x4 blocks: rows 0..3 and rows 4..7
+  __device__ static inline void run(const u32x4 (&r)[8], u32x4 (&c)[8]) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int d = 0; d < 4; ++d) c[h * 4 + j][d] = r[h * 4 + d][j];
+  }
+};
+
+// ---- operand loaders -----------------------------------------------------------------------------
+// A "tile operand" is 256 rows x one K slab.  fetch() pulls the slab into 8 x 16-byte registers,
+// commit() writes them to LDS.
+
+// k-contiguous rows: thread -> chunk (tid & 7) of rows (tid >> 3) + 32 i.
+template <typename T>
+struct KContigLoader {
+  static constexpr int V = ElemTraits<T>::kVec;
+  const T *base;
+  long long row_off[8];  // element offset of each of this thread's rows
+  int chunk, Kd;
+  u32x4 regs[8];
+
+  __device__ inline void fetch(int k0) {
+    int k = k0 + chunk * V;
+    bool ok = k < Kd;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      u32x4 v = {0, 0, 0, 0};
+      if (ok) v = *(const u32x4 *)(base + row_off[i] + k);
+      regs[i] = v;
+    }
+  }
+  __device__ inline void commit(char *lds, int tid) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int row = (tid >> 3) + 32 * i;
+      *(u32x4 *)(lds + lds_chunk_off(row, chunk)) = regs[i];
+    }
+  }
+};
+
+// Operand stored as [k][row] with `row` contiguous: element (k, r) at base + k * ld + r.
+// thread -> k-block (lane & 7), row blocks wave*8 + (lane >> 3) (+32 for the second fp32 block).
+template <typename T, bool GLU_ROWS>
+struct TransposedLoader {
+  static constexpr int V = ElemTraits<T>::kVec;
+  static constexpr int NB = 8 / V;  // row blocks per thread (1 for 16-bit, 2 for fp32)
+  const T *base;                    // already offset to (k = 0, row = tile row 0)
+  long long ld;
+  int kb, rb, k_valid, r_valid;
+  u32x4 regs[8];
+
+  __device__ inline void fetch(int k0) {
+#pragma unroll
+    for (int h = 0; h < NB; ++h) {
+      int r = (rb + 32 * h) * V;
+      bool r_ok = r < r_valid;
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        int k = k0 + kb * V + i;
+        u32x4 v = {0, 0, 0, 0};
+        if (r_ok && k < k_valid) v = *(const u32x4 *)(base + (long long)k * ld + r);
+        regs[h * V + i] = v;
+      }
+    }
+  }
+  // LDS row of tile column r: with GLU_ROWS the interleaved (gate, up) columns of each 128-column
+  // wave range are split into 64 gate rows followed by 64 up rows.
+  __device__ static inline int lds_row(int r) {
+    if (!GLU_ROWS) return r;
+    int x = r & 127;
+    return (r & ~127) | ((x & 1) << 6) | (x >> 1);
+  }
+  __device__ inline void commit(char *lds) {
+    u32x4 cols[8];
+    BlockTranspose<sizeof(T)>::run(regs, cols);
+#pragma unroll
+    for (int h = 0; h < NB; ++h)
+#pragma unroll
+      for (int j = 0; j < V; ++j) {
+        int row = lds_row((rb + 32 * h) * V + j);
+        *(u32x4 *)(lds + lds_chunk_off(row, kb)) = cols[h * V + j];
+      }
+  }
+};
+
+template <typename T, int A_KIND, int B_KIND, int EPI, int PROB, bool GATHER>
+__global__ __launch_bounds__(kGemmThreads) void grouped_gemm_kernel(const GemmArgs args) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  constexpr int BK = kRowBytes / (int)sizeof(T);
+  constexpr bool GLU_ROWS = EPI == EPI_GLU;
+  static_assert(!(EPI == EPI_GLU) || B_KIND == OP_TRANSPOSED, "GLU epilogue expects [K,N] weights");
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // ---- which tile -------------------------------------------------------------------------------
+  int expert, row0, rows_valid, col_tile, k_len;
+  long long a_first = 0;  // PROB_WGRAD: first k row of the expert
+  int m0 = 0;             // PROB_WGRAD: first output row of this tile
+  {
+    int n_row_tiles = (PROB == PROB_ROWS) ? args.sched[0] : args.E * args.n_row_tiles_wgrad;
+    int total = n_row_tiles * args.n_col_tiles;
+    int total8 = (total + kXcds - 1) / kXcds * kXcds;
+    int b = blockIdx.x;
+    if (b >= total8) return;
+    int L = (b % kXcds) * (total8 / kXcds) + b / kXcds;
+    if (L >= total) return;
+    if (PROB == PROB_ROWS) {
+      const int *tiles = args.sched + kSchedHeader;
+      int t0 = L / args.n_col_tiles;
+      int gfirst = tiles[8 * t0 + 3], gcount = tiles[8 * t0 + 4];
+      int local = L - gfirst * args.n_col_tiles;
+      col_tile = local / gcount;
+      const int *te = tiles + 8 * (gfirst + local % gcount);
+      expert = te[0]; row0 = te[1]; rows_valid = te[2];
+      k_len = args.Kd;
+    } else {
+      int per_expert = args.n_row_tiles_wgrad * args.n_col_tiles;
+      expert = L / per_expert;
+      int local = L - expert * per_expert;
+      col_tile = local / args.n_row_tiles_wgrad;
+      m0 = (local % args.n_row_tiles_wgrad) * kBM;
+      row0 = 0;
+      rows_valid = min(kBM, args.Md - m0);
+      k_len = min(args.counts[expert], args.capacity);
+      a_first = args.offsets[expert];
+    }
+  }
+  const int n0 = col_tile * kBN;
+
+  // ---- loaders ------------------------------------------------------------------------------------
+  KContigLoader<T> a_k;
+  TransposedLoader<T, false> a_t;
+  KContigLoader<T> b_k;
+  TransposedLoader<T, GLU_ROWS> b_t;
+  if (A_KIND == OP_KCONTIG) {
+    a_k.base = (const T *)args.A;
+    a_k.chunk = tid & 7;
+    a_k.Kd = k_len;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int r = min((tid >> 3) + 32 * i, rows_valid - 1);
+      long long src = row0 + r;
+      if (GATHER) src = args.a_rows[row0 + r] / args.a_div;
+      a_k.row_off[i] = src * args.lda;
+    }
+  } else {
+    a_t.base = (const T *)args.A + a_first * args.lda + m0;
+    a_t.ld = args.lda;
+    a_t.kb = lane & 7;
+    a_t.rb = wave * 8 + (lane >> 3);
+    a_t.k_valid = k_len;
+    a_t.r_valid = rows_valid;
+  }
+  if (B_KIND == OP_KCONTIG) {
+    // B element (k, n) at B[expert][n][k]: rows are output columns
+    b_k.base = (const T *)args.B + (long long)expert * args.b_expert_stride;
+    b_k.chunk = tid & 7;
+    b_k.Kd = k_len;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int n = min(n0 + (tid >> 3) + 32 * i, args.Nd - 1);
+      b_k.row_off[i] = (long long)n * args.ldb;
+    }
+  } else {
+    if (PROB == PROB_ROWS)
+      b_t.base = (const T *)args.B + (long long)expert * args.b_expert_stride + n0;
+    else
+      b_t.base = (const T *)args.B + a_first * args.ldb + n0;
+    b_t.ld = args.ldb;
+    b_t.kb = lane & 7;
+    b_t.rb = wave * 8 + (lane >> 3);
+    b_t.k_valid = k_len;
+    b_t.r_valid = args.Nd - n0;
+  }
+
+  // LDS: stage 0 = {A, B}, stage 1 = {A, B}
+
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < 4; ++ni)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
+
+  // 32-row blocks of the tile are dealt alternately to the two wave rows; blocks past the valid
+  // rows are skipped.
+  const int n_blocks32 = (rows_valid + 31) >> 5;
+  const int n_mi = (n_blocks32 - wm + 1) >> 1;
+  const int n_slabs = (k_len + BK - 1) / BK;
+
+  auto fetch = [&](int s) {
+    if (A_KIND == OP_KCONTIG) a_k.fetch(s * BK); else a_t.fetch(s * BK);
+    if (B_KIND == OP_KCONTIG) b_k.fetch(s * BK); else b_t.fetch(s * BK);
+  };
+  auto commit = [&](int buf) {
+    char *tA = lds + buf * (2 * kTileBytes), *tB = tA + kTileBytes;
+    if (A_KIND == OP_KCONTIG) a_k.commit(tA, tid); else a_t.commit(tA);
+    if (B_KIND == OP_KCONTIG) b_k.commit(tB, tid); else b_t.commit(tB);
+  };
+
+  if (n_slabs > 0) {
+    fetch(0);
+    commit(0);
+  }
+  __syncthreads();
+
+  for (int s = 0; s < n_slabs; ++s) {
+    const int buf = s & 1;
+    if (s + 1 < n_slabs) fetch(s + 1);
+    const char *tA = lds + buf * (2 * kTileBytes), *tB = tA + kTileBytes;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const int chunk = ks * 2 + (lane >> 5);
+      u32x4 bf[4];
+#pragma unroll
+      for (int ni = 0; ni < 4; ++ni) {
+        int row = wn * 128 + ni * 32 + (lane & 31);
+        bf[ni] = *(const u32x4 *)(tB + lds_chunk_off(row, chunk));
+      }
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) {
+        if (mi < n_mi) {
+          int row = (mi * 2 + wm) * 32 + (lane & 31);
+          u32x4 af = *(const u32x4 *)(tA + lds_chunk_off(row, chunk));
+#pragma unroll
+          for (int ni = 0; ni < 4; ++ni) Mma<T>::run(af, bf[ni], acc[mi][ni]);
+        }
+      }
+    }
+    if (s + 1 < n_slabs) commit(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue -------------------------------------------------------------------------------------
+  // acc[mi][ni][v]: tile row (mi*2+wm)*32 + 8*(v/4) + 4*(lane/32) + v%4, LDS column row wn*128 + ni*32 + lane%32
+  const int lcol = lane & 31;
+  const int rsub = (lane >> 5) * 4;
+  if (EPI == EPI_STORE) {
+    T *C = (T *)args.C;
+    long long c_base = (PROB == PROB_WGRAD) ? (long long)expert * args.c_expert_stride : 0;
+#pragma unroll
+    for (int ni = 0; ni < 4; ++ni) {
+      int col = n0 + wn * 128 + ni * 32 + lcol;
+      bool col_ok = col < args.Nd;
+      float bias = 0.0f;
+      if (args.bias != nullptr && col_ok)
+        bias = ElemTraits<T>::to_f32(((const T *)args.bias)[(long long)expert * args.Nd + col]);
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) {
+        if (mi < n_mi) {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            int r = (mi * 2 + wm) * 32 + 8 * (v >> 2) + rsub + (v & 3);
+            if (col_ok && r < rows_valid) {
+              long long orow = (PROB == PROB_WGRAD) ? (m0 + r) : (row0 + r);
+              C[c_base + orow * args.ldc + col] = ElemTraits<T>::from_f32(acc[mi][ni][v] + bias);
+            }
+          }
+        }
+      }
+    }
+  } else {
+    // gate columns live in ni = 0,1 and the matching up columns in ni = 2,3
+    T *C = (T *)args.C;
+    T *P = (T *)args.C2;
+#pragma unroll
+    for (int np = 0; np < 2; ++np) {
+      int pair = (n0 + wn * 128) / 2 + np * 32 + lcol;  // index of the (gate, up) pair = act column
+      bool col_ok = 2 * pair + 1 < args.Nd;
+      float bg = 0.0f, bu = 0.0f;
+      if (EPI == EPI_GLU && args.bias != nullptr && col_ok) {
+        const T *bp = (const T *)args.bias + (long long)expert * args.Nd + 2 * pair;
+        bg = ElemTraits<T>::to_f32(bp[0]);
+        bu = ElemTraits<T>::to_f32(bp[1]);
+      }
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) {
+        if (mi < n_mi) {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            int r = (mi * 2 + wm) * 32 + 8 * (v >> 2) + rsub + (v & 3);
+            if (col_ok && r < rows_valid) {
+              long long orow = row0 + r;
+              if (EPI == EPI_GLU) {
+                float G = acc[mi][np][v] + bg, U = acc[mi][np + 2][v] + bu;
+                C[orow * args.ldc + pair] = ElemTraits<T>::from_f32(glu_forward(G, U));
+                if (P != nullptr) {
+                  P[orow * args.Nd + 2 * pair] = ElemTraits<T>::from_f32(G);
+                  P[orow * args.Nd + 2 * pair + 1] = ElemTraits<T>::from_f32(U);
+                }
+              }
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+// GLU backward on rows: d_act [rows, I] and the stored pre-activations [rows, 2I] give the
+// interleaved (gate, up) pre-activation gradients [rows, 2I] (csrc/experts_backward.cu:285-305).
+template <typename T>
+__global__ __launch_bounds__(256) void glu_backward_rows_kernel(const T *__restrict__ d_act,
+                                                                const T *__restrict__ pre,
+                                                                T *__restrict__ d_pre, long long n_pairs) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  long long stride = (long long)gridDim.x * blockDim.x;
+  for (; i < n_pairs; i += stride) {
+    float G = ElemTraits<T>::to_f32(pre[2 * i]), U = ElemTraits<T>::to_f32(pre[2 * i + 1]);
+    float dG, dU;
+    glu_backward(G, U, ElemTraits<T>::to_f32(d_act[i]), dG, dU);
+    d_pre[2 * i] = ElemTraits<T>::from_f32(dG);
+    d_pre[2 * i + 1] = ElemTraits<T>::from_f32(dU);
+  }
+}
+
+// Experts that own no kept rows need no special case in the weight-gradient product: k_len = 0
+// leaves the accumulators at zero and the epilogue stores them.
+
+template <typename T, int A_KIND, int B_KIND, int EPI, int PROB, bool GATHER>
+static int launch_gemm(const GemmArgs &args, int max_row_tiles, hipStream_t stream) {
+  auto kernel = grouped_gemm_kernel<T, A_KIND, B_KIND, EPI, PROB, GATHER>;
+  static bool attr_done = false;  // benign race: the attribute call is idempotent
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(MaxDynamicSharedMemorySize=%d): %s", kGemmLds, hipGetErrorString(e));
+      return (int)e;
+    }
+    attr_done = true;
+  }
+  long long total = (long long)max_row_tiles * args.n_col_tiles;
+  if (total <= 0) return 0;
+  total = (total + kXcds - 1) / kXcds * kXcds;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(kGemmThreads), kGemmLds, stream, args);
+  return check_launch("grouped_gemm_kernel");
+}
+
+template <typename T>
+int gemm_gate_up(const void *x, const int *sorted_idx, const void *w, const void *bias, void *act, void *pre,
+                 const void *sched, int N, int K, int E, int H, int I, hipStream_t stream) {
+  GemmArgs a = {};
+  a.A = x; a.B = w; a.bias = bias; a.C = act; a.C2 = pre;
+  a.a_rows = sorted_idx; a.a_div = K; a.sched = (const int *)sched;
+  a.Kd = H; a.Nd = 2 * I; a.lda = H; a.ldb = 2 * I; a.ldc = I;
+  a.b_expert_stride = (long long)H * 2 * I;
+  a.n_col_tiles = ceil_div(2 * I, kBN);
+  a.N = N; a.E = E;
+  return launch_gemm<T, OP_KCONTIG, OP_TRANSPOSED, EPI_GLU, PROB_ROWS, true>(a, sched_max_row_tiles(N, E), stream);
+}
+
+template <typename T>
+int gemm_down(const void *act, const void *w, const void *bias, void *y, const void *sched, int N, int E, int H,
+              int I, hipStream_t stream) {
+  GemmArgs a = {};
+  a.A = act; a.B = w; a.bias = bias; a.C = y; a.sched = (const int *)sched;
+  a.Kd = I; a.Nd = H; a.lda = I; a.ldb = H; a.ldc = H;
+  a.b_expert_stride = (long long)I * H;
+  a.n_col_tiles = ceil_div(H, kBN);
+  a.N = N; a.E = E;
+  return launch_gemm<T, OP_KCONTIG, OP_TRANSPOSED, EPI_STORE, PROB_ROWS, false>(a, sched_max_row_tiles(N, E), stream);
+}
+
+// d_out[p,:] = g[p,:] . W[e]^T with W[e] = [n_out, k] row-major, i.e. k-contiguous "B rows".
+template <typename T>
+int gemm_dgrad(const void *g, const void *w, void *d_out, const void *sched, int N, int E, int Kd, int Nd,
+               hipStream_t stream) {
+  GemmArgs a = {};
+  a.A = g; a.B = w; a.C = d_out; a.sched = (const int *)sched;
+  a.Kd = Kd; a.Nd = Nd; a.lda = Kd; a.ldb = Kd; a.ldc = Nd;
+  a.b_expert_stride = (long long)Nd * Kd;
+  a.n_col_tiles = ceil_div(Nd, kBN);
+  a.N = N; a.E = E;
+  return launch_gemm<T, OP_KCONTIG, OP_KCONTIG, EPI_STORE, PROB_ROWS, false>(a, sched_max_row_tiles(N, E), stream);
+}
+
+// dW[e] = L_e^T . R_e over the expert's kept rows: L [rows, Md], R [rows, Nd], dW [E, Md, Nd].
+template <typename T>
+int gemm_wgrad(const void *L, const void *R, void *dW, const int *counts, const int *offsets, int capacity, int E,
+               int Md, int Nd, hipStream_t stream) {
+  GemmArgs a = {};
+  a.A = L; a.B = R; a.C = dW; a.counts = counts; a.offsets = offsets; a.capacity = capacity;
+  a.Md = Md; a.Nd = Nd; a.lda = Md; a.ldb = Nd; a.ldc = Nd;
+  a.c_expert_stride = (long long)Md * Nd;
+  a.n_col_tiles = ceil_div(Nd, kBN);
+  a.n_row_tiles_wgrad = ceil_div(Md, kBM);
+  a.E = E;
+  return launch_gemm<T, OP_TRANSPOSED, OP_TRANSPOSED, EPI_STORE, PROB_WGRAD, false>(a, E * a.n_row_tiles_wgrad, stream);
+}
+
+template <typename T>
+int glu_backward_rows(const void *d_act, const void *pre, void *d_pre, long long n_pairs, hipStream_t stream) {
+  if (n_pairs == 0) return 0;
+  long long blocks = (n_pairs + 255) / 256;
+  if (blocks > 256 * 32) blocks = 256 * 32;
+  hipLaunchKernelGGL(glu_backward_rows_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, (const T *)d_act,
+                     (const T *)pre, (T *)d_pre, n_pairs);
+  return check_launch("glu_backward_rows_kernel");
+}
+
+#define YAMOE_INSTANTIATE_GEMM(T)                                                                                   \
+  template int gemm_gate_up<T>(const void *, const int *, const void *, const void *, void *, void *, const void *, \
+                               int, int, int, int, int, hipStream_t);                                               \
+  template int gemm_down<T>(const void *, const void *, const void *, void *, const void *, int, int, int, int,     \
+                            hipStream_t);                                                                           \
+  template int gemm_dgrad<T>(const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);    \
+  template int gemm_wgrad<T>(const void *, const void *, void *, const int *, const int *, int, int, int, int,      \
+                             hipStream_t);                                                                          \
+  template int glu_backward_rows<T>(const void *, const void *, void *, long long, hipStream_t);
+YAMOE_INSTANTIATE_GEMM(float)
+YAMOE_INSTANTIATE_GEMM(bf16_t)
+YAMOE_INSTANTIATE_GEMM(f16_t)
+
+}  // namespace yamoe

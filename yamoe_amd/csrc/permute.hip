@@ -1,0 +1,257 @@
+// Row movers of the expert layer: the token permute (expert-contiguous gather of rows) and the
+// routing-weighted combine that brings expert outputs back to token order.
+//
+// Both are pure HBM streaming: one wavefront moves one row in 16-byte chunks per lane, so every
+// request is a full coalesced segment.  The combine replaces the reference's atomic scatter-add
+// (csrc/scatter.cu:66-108): each output row is owned by one wave, which sums the K expert rows of
+// its token through the inverse permutation in fp32 in slot order and rounds once.
+#include "common.h"
+
+namespace yamoe {
+
+constexpr int kRowThreads = 256;
+constexpr int kRowWaves = kRowThreads / kWave;
+
+// x_perm[p,:] = x[sorted_idx[p] / K,:]   (csrc/gather.cu:6-66 without the padding rows)
+template <typename T>
+__global__ __launch_bounds__(kRowThreads) void permute_kernel(const T *__restrict__ x,
+                                                              const int *__restrict__ sorted_idx,
+                                                              T *__restrict__ x_perm, int N, int K,
+                                                              int H) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = blockIdx.x * kRowWaves + threadIdx.x / kWave;
+  const int n_waves = gridDim.x * kRowWaves;
+  constexpr int V = ElemTraits<T>::kVec;
+  const bool vec_ok = (H % V) == 0;
+  for (int p = wave; p < N; p += n_waves) {
+    int tok = sorted_idx[p] / K;
+    const T *src = x + (size_t)tok * H;
+    T *dst = x_perm + (size_t)p * H;
+    if (vec_ok) {
+      const u32x4 *s4 = (const u32x4 *)src;
+      u32x4 *d4 = (u32x4 *)dst;
+      for (int c = lane; c < H / V; c += kWave) d4[c] = s4[c];
+    } else {
+      for (int c = lane; c < H; c += kWave) dst[c] = src[c];
+    }
+  }
+}
+
+template <typename T, bool I64>
+__device__ inline float slot_weight(const T *rw, const void *idx, int t, int k, int K, int E,
+                                    int rw_cols) {
+  if (rw == nullptr) return 1.0f;
+  if (rw_cols == K && rw_cols != E) return ElemTraits<T>::to_f32(rw[(size_t)t * K + k]);
+  long long e = I64 ? ((const long long *)idx)[(size_t)t * K + k]
+                    : (long long)((const int *)idx)[(size_t)t * K + k];
+  if (e < 0 || e >= E) return 0.0f;
+  return ElemTraits<T>::to_f32(rw[(size_t)t * E + e]);
+}
+
+// out[t,:] = sum_k w(t,k) * y_perm[inv_pos[t*K+k],:]
+template <typename T, bool I64>
+__global__ __launch_bounds__(kRowThreads) void combine_kernel(
+    const T *__restrict__ y_perm, const int *__restrict__ inv_pos, const void *__restrict__ idx,
+    const T *__restrict__ rw, int rw_cols, T *__restrict__ out, int Tn, int K, int E, int H) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = blockIdx.x * kRowWaves + threadIdx.x / kWave;
+  const int n_waves = gridDim.x * kRowWaves;
+  constexpr int V = ElemTraits<T>::kVec;
+  const bool vec_ok = (H % V) == 0;
+  for (int t = wave; t < Tn; t += n_waves) {
+    T *dst = out + (size_t)t * H;
+    if (vec_ok) {
+      for (int c = lane; c < H / V; c += kWave) {
+        float acc[V];
+#pragma unroll
+        for (int j = 0; j < V; ++j) acc[j] = 0.0f;
+        for (int k = 0; k < K; ++k) {
+          int pos = inv_pos[(size_t)t * K + k];
+          if (pos < 0) continue;
+          float w = slot_weight<T, I64>(rw, idx, t, k, K, E, rw_cols);
+          u32x4 raw = ((const u32x4 *)(y_perm + (size_t)pos * H))[c];
+          const T *v = (const T *)&raw;
+#pragma unroll
+          for (int j = 0; j < V; ++j) acc[j] += w * ElemTraits<T>::to_f32(v[j]);
+        }
+        u32x4 o;
+        T *ov = (T *)&o;
+#pragma unroll
+        for (int j = 0; j < V; ++j) ov[j] = ElemTraits<T>::from_f32(acc[j]);
+        ((u32x4 *)dst)[c] = o;
+      }
+    } else {
+      for (int c = lane; c < H; c += kWave) {
+        float acc = 0.0f;
+        for (int k = 0; k < K; ++k) {
+          int pos = inv_pos[(size_t)t * K + k];
+          if (pos < 0) continue;
+          float w = slot_weight<T, I64>(rw, idx, t, k, K, E, rw_cols);
+          acc += w * ElemTraits<T>::to_f32(y_perm[(size_t)pos * H + c]);
+        }
+        dst[c] = ElemTraits<T>::from_f32(acc);
+      }
+    }
+  }
+}
+
+// Backward of the combine (csrc/experts_backward.cu:37-89) in sorted-row order:
+//   g_y_perm[p,:] = grad_out[tok,:] * w(tok,slot)          for kept rows p
+//   d_sel[flat]   = <grad_out[tok,:], y_perm[p,:]>         (fp32 wave-parallel dot)
+// and the dense routing gradient d_routing[tok, expert] = d_sel (zero elsewhere is the caller's
+// fill).  Dropped slots get no row and a zero gradient.
+template <typename T, bool I64>
+__global__ __launch_bounds__(kRowThreads) void combine_backward_kernel(
+    const T *__restrict__ grad_out, const T *__restrict__ y_perm, const int *__restrict__ sorted_idx,
+    const int *__restrict__ inv_pos, const void *__restrict__ idx, const T *__restrict__ rw,
+    int rw_cols, T *__restrict__ g_y_perm, T *__restrict__ d_routing, int N, int K, int E, int H) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = blockIdx.x * kRowWaves + threadIdx.x / kWave;
+  const int n_waves = gridDim.x * kRowWaves;
+  for (int p = wave; p < N; p += n_waves) {
+    int flat = sorted_idx[p];
+    if (inv_pos[flat] != p) continue;  // dropped or invalid expert id
+    int t = flat / K, k = flat - t * K;
+    float w = slot_weight<T, I64>(rw, idx, t, k, K, E, rw_cols);
+    const T *g = grad_out + (size_t)t * H;
+    const T *y = y_perm + (size_t)p * H;
+    T *o = g_y_perm + (size_t)p * H;
+    float dot = 0.0f;
+    for (int c = lane; c < H; c += kWave) {
+      float gv = ElemTraits<T>::to_f32(g[c]);
+      dot += gv * ElemTraits<T>::to_f32(y[c]);
+      o[c] = ElemTraits<T>::from_f32(gv * w);
+    }
+    for (int d = kWave / 2; d > 0; d >>= 1) dot += __shfl_xor(dot, d);
+    if (lane == 0) {
+      if (rw_cols == K && rw_cols != E) {
+        d_routing[(size_t)t * K + k] = ElemTraits<T>::from_f32(dot);
+      } else {
+        long long e = I64 ? ((const long long *)idx)[flat] : (long long)((const int *)idx)[flat];
+        d_routing[(size_t)t * E + e] = ElemTraits<T>::from_f32(dot);
+      }
+    }
+  }
+}
+
+// Column sums over each expert's kept rows: out[e, c] = sum_{rows p of e} src[p, c]
+// (d_down_proj_bias and d_gate_up_proj_bias, csrc/experts_backward.cu:277, 308).
+// grid (E, ceil(cols / kRowThreads)); a thread owns one column and walks the rows in order.
+template <typename T>
+__global__ __launch_bounds__(kRowThreads) void expert_colsum_kernel(const T *__restrict__ src,
+                                                                    const int *__restrict__ counts,
+                                                                    const int *__restrict__ offsets,
+                                                                    int capacity, T *__restrict__ out,
+                                                                    int cols) {
+  const int e = blockIdx.x;
+  const int c = blockIdx.y * kRowThreads + threadIdx.x;
+  if (c >= cols) return;
+  int first = offsets[e], kept = min(counts[e], capacity);
+  float acc = 0.0f;
+  for (int r = 0; r < kept; ++r) acc += ElemTraits<T>::to_f32(src[(size_t)(first + r) * cols + c]);
+  out[(size_t)e * cols + c] = ElemTraits<T>::from_f32(acc);
+}
+
+template <typename T>
+int launch_permute(const void *x, const int *sorted_idx, void *x_perm, int N, int K, int H,
+                   hipStream_t stream) {
+  if (N == 0) return 0;
+  int blocks = min(ceil_div(N, kRowWaves), 256 * 16);
+  hipLaunchKernelGGL(permute_kernel<T>, dim3(blocks), dim3(kRowThreads), 0, stream, (const T *)x,
+                     sorted_idx, (T *)x_perm, N, K, H);
+  return check_launch("permute_kernel");
+}
+
+template <typename T>
+int launch_combine(const void *y_perm, const int *inv_pos, const void *idx, int idx_i64,
+                   const void *rw, int rw_cols, void *out, int Tn, int K, int E, int H,
+                   hipStream_t stream) {
+  if (Tn == 0) return 0;
+  int blocks = min(ceil_div(Tn, kRowWaves), 256 * 16);
+  if (idx_i64)
+    hipLaunchKernelGGL((combine_kernel<T, true>), dim3(blocks), dim3(kRowThreads), 0, stream,
+                       (const T *)y_perm, inv_pos, idx, (const T *)rw, rw_cols, (T *)out, Tn, K, E, H);
+  else
+    hipLaunchKernelGGL((combine_kernel<T, false>), dim3(blocks), dim3(kRowThreads), 0, stream,
+                       (const T *)y_perm, inv_pos, idx, (const T *)rw, rw_cols, (T *)out, Tn, K, E, H);
+  return check_launch("combine_kernel");
+}
+
+template <typename T>
+int launch_combine_backward(const void *grad_out, const void *y_perm, const int *sorted_idx,
+                            const int *inv_pos, const void *idx, int idx_i64, const void *rw,
+                            int rw_cols, void *g_y_perm, void *d_routing, int N, int K, int E, int H,
+                            hipStream_t stream) {
+  if (N == 0) return 0;
+  int blocks = min(ceil_div(N, kRowWaves), 256 * 16);
+  if (idx_i64)
+    hipLaunchKernelGGL((combine_backward_kernel<T, true>), dim3(blocks), dim3(kRowThreads), 0, stream,
+                       (const T *)grad_out, (const T *)y_perm, sorted_idx, inv_pos, idx, (const T *)rw,
+                       rw_cols, (T *)g_y_perm, (T *)d_routing, N, K, E, H);
+  else
+    hipLaunchKernelGGL((combine_backward_kernel<T, false>), dim3(blocks), dim3(kRowThreads), 0, stream,
+                       (const T *)grad_out, (const T *)y_perm, sorted_idx, inv_pos, idx, (const T *)rw,
+                       rw_cols, (T *)g_y_perm, (T *)d_routing, N, K, E, H);
+  return check_launch("combine_backward_kernel");
+}
+
+template <typename T>
+int launch_expert_colsum(const void *src, const int *counts, const int *offsets, int capacity,
+                         void *out, int E, int cols, hipStream_t stream) {
+  hipLaunchKernelGGL(expert_colsum_kernel<T>, dim3(E, ceil_div(cols, kRowThreads)), dim3(kRowThreads), 0,
+                     stream, (const T *)src, counts, offsets, capacity, (T *)out, cols);
+  return check_launch("expert_colsum_kernel");
+}
+
+#define YAMOE_INSTANTIATE_ROWS(T)                                                                       \
+  template int launch_permute<T>(const void *, const int *, void *, int, int, int, hipStream_t);        \
+  template int launch_combine<T>(const void *, const int *, const void *, int, const void *, int,       \
+                                 void *, int, int, int, int, hipStream_t);                              \
+  template int launch_combine_backward<T>(const void *, const void *, const int *, const int *,        \
+                                          const void *, int, const void *, int, void *, void *, int,   \
+                                          int, int, int, hipStream_t);                                  \
+  template int launch_expert_colsum<T>(const void *, const int *, const int *, int, void *, int, int,  \
+                                       hipStream_t);
+YAMOE_INSTANTIATE_ROWS(float)
+YAMOE_INSTANTIATE_ROWS(bf16_t)
+YAMOE_INSTANTIATE_ROWS(f16_t)
+
+}  // namespace yamoe
+
+using namespace yamoe;
+
+#define YAMOE_DISPATCH(dtype, CALL)                                \
+  switch (dtype) {                                                 \
+    case YAMOE_F32: { typedef float T; return CALL; }              \
+    case YAMOE_BF16: { typedef bf16_t T; return CALL; }            \
+    case YAMOE_F16: { typedef f16_t T; return CALL; }              \
+    default: set_error("unknown dtype %d", dtype); return YAMOE_E_DTYPE; \
+  }
+
+extern "C" int yamoe_permute(const void *x, const int32_t *sorted_idx, void *x_perm, int32_t N,
+                             int32_t K, int32_t H, int32_t dtype, void *stream) {
+  if (N < 0 || K <= 0 || H <= 0 || (N > 0 && (!x || !sorted_idx || !x_perm))) {
+    set_error("yamoe_permute: bad argument");
+    return YAMOE_E_ARG;
+  }
+  YAMOE_DISPATCH(dtype, launch_permute<T>(x, sorted_idx, x_perm, N, K, H, (hipStream_t)stream));
+}
+
+extern "C" int yamoe_combine(const void *y_perm, const int32_t *inv_pos, const void *router_indices,
+                             int32_t idx_i64, const void *routing_weights, int32_t rw_cols, void *out,
+                             int32_t T_, int32_t K, int32_t E, int32_t H, int32_t dtype, void *stream) {
+  if (T_ < 0 || K <= 0 || H <= 0 || E <= 0 || (T_ > 0 && (!y_perm || !inv_pos || !out))) {
+    set_error("yamoe_combine: bad argument");
+    return YAMOE_E_ARG;
+  }
+  if (routing_weights && rw_cols != E && rw_cols != K) {
+    set_error("yamoe_combine: routing_weights must have E or K columns (got %d)", rw_cols);
+    return YAMOE_E_ARG;
+  }
+  if (routing_weights && rw_cols == E && !router_indices) {
+    set_error("yamoe_combine: dense routing_weights need router_indices");
+    return YAMOE_E_ARG;
+  }
+  YAMOE_DISPATCH(dtype, launch_combine<T>(y_perm, inv_pos, router_indices, idx_i64, routing_weights, rw_cols,
+                                          out, T_, K, E, H, (hipStream_t)stream));
+}

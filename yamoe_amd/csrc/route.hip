@@ -1,0 +1,363 @@
+// Routing for the expert layer: a stable counting sort of the N = T*K (token, slot) assignments by
+// expert id, the per-expert counts and exclusive offsets, the inverse permutation, and the work
+// lists the expert GEMM kernels walk.
+//
+// Replaces cub::DeviceRadixSort::SortPairs (csrc/sort.cu:17-91) and bincount_cumsum_kernel
+// (csrc/bincount_cumsum.cu:7-56).  The keys have ceil(log2 E) meaningful bits, so one counting pass
+// is enough: the input is cut into contiguous segments, one per wavefront; each wave histograms
+// its segment, a scan turns (expert-major, segment-minor) counts into write cursors, and each wave
+// then walks its segment in order and places every element at cursor[expert] + (number of equal
+// keys in lower lanes of the same 64-element step), found with wavefront ballots.  Walking in order
+// and ranking by lane keeps equal keys in input order, i.e. the sort is stable.
+#include "common.h"
+
+namespace yamoe {
+
+constexpr int kRouteThreads = 1024;
+constexpr int kRouteWaves = kRouteThreads / kWave;
+constexpr int kRouteMaxBuckets = 769;    // E + 1 must not exceed this (keeps dynamic LDS under 64 KB)
+constexpr int kSingleBlockMaxN = 32768;  // above this the three-kernel form is used
+
+template <bool I64>
+__device__ inline int load_key(const void *idx, int i, int E) {
+  long long v = I64 ? ((const long long *)idx)[i] : (long long)((const int *)idx)[i];
+  // ids outside [0,E) go to bucket E, after every valid expert
+  return (v < 0 || v >= E) ? E : (int)v;
+}
+template <bool I64>
+__device__ inline int load_raw(const void *idx, int i) {
+  return I64 ? (int)((const long long *)idx)[i] : ((const int *)idx)[i];
+}
+
+// Lanes of this wave whose key equals mine (only among lanes with `active`).
+__device__ inline uint64_t match_key(int key, bool active, int key_bits) {
+  uint64_t peers = __ballot(active);
+  for (int b = 0; b < key_bits; ++b) {
+    bool bit = (key >> b) & 1;
+    uint64_t m = __ballot(active && bit);
+    peers &= bit ? m : ~m;
+  }
+  return peers;
+}
+
+__device__ inline int bits_for(int buckets) {
+  int b = 0;
+  while ((1 << b) < buckets) ++b;
+  return b;
+}
+
+// Histogram of one wave's segment [seg_begin, seg_end) into `hist` (LDS or global, zeroed by caller).
+template <bool I64>
+__device__ inline void wave_histogram(const void *idx, int seg_begin, int seg_end, int E,
+                                      int *hist_lds) {
+  const int lane = threadIdx.x & (kWave - 1);
+  for (int i = seg_begin + lane; i < seg_end; i += kWave) {
+    int key = load_key<I64>(idx, i, E);
+    atomicAdd(&hist_lds[key], 1);
+  }
+}
+
+// Walk one segment in order and place its elements.  `cursor` (LDS, private to this wave) holds
+// the next free sorted position per bucket.
+template <bool I64>
+__device__ inline void wave_place(const void *idx, int seg_begin, int seg_end, int E, int capacity,
+                                  volatile int *cursor, const int *offsets_lds,
+                                  int *sorted_expert, int *sorted_idx, int *inv_pos) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int key_bits = bits_for(E + 1);
+  const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  for (int base = seg_begin; base < seg_end; base += kWave) {
+    int i = base + lane;
+    bool active = i < seg_end;
+    int key = active ? load_key<I64>(idx, i, E) : 0;
+    uint64_t peers = match_key(key, active, key_bits);
+    int rank = __popcll(peers & lt_mask);
+    int start = 0;
+    if (active) start = cursor[key];
+    __builtin_amdgcn_wave_barrier();
+    if (active) {
+      int pos = start + rank;
+      sorted_expert[pos] = load_raw<I64>(idx, i);
+      sorted_idx[pos] = i;
+      bool kept = key < E && (pos - offsets_lds[key]) < capacity;
+      inv_pos[i] = kept ? pos : -1;
+      if (rank == 0) cursor[key] = start + __popcll(peers);
+    }
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+  }
+}
+
+// Exclusive scan over buckets of `total` into `offsets` (both LDS), done by the whole block.
+// offsets[b] for b in [0, buckets]; offsets[buckets] = N.
+__device__ inline void block_exclusive_scan(const int *total, int *offsets, int buckets,
+                                            int *scratch /* kRouteWaves + 1 ints */) {
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  int carry = 0;
+  for (int base = 0; base < buckets; base += blockDim.x) {
+    int b = base + tid;
+    int v = (b < buckets) ? total[b] : 0;
+    // inclusive scan inside the wave
+    int x = v;
+    for (int d = 1; d < kWave; d <<= 1) {
+      int y = __shfl_up(x, d);
+      if (lane >= d) x += y;
+    }
+    if (lane == kWave - 1) scratch[wave] = x;
+    __syncthreads();
+    int wave_off = 0;
+    for (int w = 0; w < wave; ++w) wave_off += scratch[w];
+    int chunk_total = 0;
+    for (int w = 0; w < (int)(blockDim.x / kWave); ++w) chunk_total += scratch[w];
+    if (b < buckets) offsets[b] = carry + wave_off + x - v;
+    carry += chunk_total;
+    __syncthreads();
+  }
+  if (tid == 0) offsets[buckets] = carry;
+  __syncthreads();
+}
+
+// ---- single-block form: everything in one launch -------------------------------------------------
+// Dynamic LDS: hist[kRouteWaves][buckets] + total[buckets] + offsets[buckets+1] + scratch.
+template <bool I64>
+__global__ __launch_bounds__(kRouteThreads) void route_single_kernel(
+    const void *idx, int N, int E, int capacity, int *sorted_expert, int *sorted_idx, int *counts,
+    int *offsets_out, int *inv_pos) {
+  extern __shared__ int lds[];
+  const int buckets = E + 1;
+  int *hist = lds;                          // [kRouteWaves][buckets]
+  int *total = hist + kRouteWaves * buckets;  // [buckets]
+  int *offs = total + buckets;              // [buckets + 1]
+  int *scratch = offs + buckets + 1;        // [kRouteWaves + 1]
+  const int tid = threadIdx.x, wave = tid / kWave;
+
+  for (int i = tid; i < kRouteWaves * buckets; i += blockDim.x) hist[i] = 0;
+  __syncthreads();
+
+  int seg = ceil_div(ceil_div(N, kRouteWaves), kWave) * kWave;
+  int seg_begin = min(wave * seg, N), seg_end = min(seg_begin + seg, N);
+  wave_histogram<I64>(idx, seg_begin, seg_end, E, hist + wave * buckets);
+  __syncthreads();
+
+  for (int b = tid; b < buckets; b += blockDim.x) {
+    int s = 0;
+    for (int w = 0; w < kRouteWaves; ++w) s += hist[w * buckets + b];
+    total[b] = s;
+  }
+  __syncthreads();
+  block_exclusive_scan(total, offs, buckets, scratch);
+
+  // cursors: hist[w][b] <- offs[b] + sum_{w' < w} hist[w'][b]
+  for (int b = tid; b < buckets; b += blockDim.x) {
+    int run = offs[b];
+    for (int w = 0; w < kRouteWaves; ++w) {
+      int c = hist[w * buckets + b];
+      hist[w * buckets + b] = run;
+      run += c;
+    }
+    if (b < E) {
+      counts[b] = total[b];
+      offsets_out[b] = offs[b];
+    } else {
+      offsets_out[E] = offs[E];
+    }
+  }
+  __syncthreads();
+
+  wave_place<I64>(idx, seg_begin, seg_end, E, capacity, hist + wave * buckets, offs, sorted_expert,
+                  sorted_idx, inv_pos);
+}
+
+// ---- three-kernel form for large N -----------------------------------------------------------
+// seg_counts is [n_seg][buckets] in global memory; one wave per segment of `seg` elements.
+template <bool I64>
+__global__ __launch_bounds__(kRouteThreads) void route_hist_kernel(const void *idx, int N, int E,
+                                                                   int seg, int *seg_counts) {
+  extern __shared__ int lds[];
+  const int buckets = E + 1;
+  const int tid = threadIdx.x, wave = tid / kWave;
+  int *hist = lds + wave * buckets;
+  for (int i = tid; i < kRouteWaves * buckets; i += blockDim.x) lds[i] = 0;
+  __syncthreads();
+  int s = blockIdx.x * kRouteWaves + wave;
+  int seg_begin = min((long long)s * seg, (long long)N), seg_end = min(seg_begin + seg, N);
+  wave_histogram<I64>(idx, seg_begin, seg_end, E, hist);
+  __syncthreads();
+  for (int i = tid; i < kRouteWaves * buckets; i += blockDim.x)
+    seg_counts[(size_t)blockIdx.x * kRouteWaves * buckets + i] = lds[i];
+}
+
+// One block: totals, offsets, then per-segment cursors written back over seg_counts.
+__global__ __launch_bounds__(kRouteThreads) void route_scan_kernel(int *seg_counts, int n_seg, int E,
+                                                                   int *counts, int *offsets_out) {
+  extern __shared__ int lds[];
+  const int buckets = E + 1;
+  int *total = lds;
+  int *offs = total + buckets;
+  int *scratch = offs + buckets + 1;
+  const int tid = threadIdx.x;
+  for (int b = tid; b < buckets; b += blockDim.x) {
+    int s = 0;
+    for (int g = 0; g < n_seg; ++g) s += seg_counts[(size_t)g * buckets + b];
+    total[b] = s;
+  }
+  __syncthreads();
+  block_exclusive_scan(total, offs, buckets, scratch);
+  for (int b = tid; b < buckets; b += blockDim.x) {
+    int run = offs[b];
+    for (int g = 0; g < n_seg; ++g) {
+      int c = seg_counts[(size_t)g * buckets + b];
+      seg_counts[(size_t)g * buckets + b] = run;
+      run += c;
+    }
+    if (b < E) {
+      counts[b] = total[b];
+      offsets_out[b] = offs[b];
+    } else {
+      offsets_out[E] = offs[E];
+    }
+  }
+}
+
+template <bool I64>
+__global__ __launch_bounds__(kRouteThreads) void route_place_kernel(
+    const void *idx, int N, int E, int capacity, int seg, const int *seg_cursors,
+    const int *offsets_in, int *sorted_expert, int *sorted_idx, int *inv_pos) {
+  extern __shared__ int lds[];
+  const int buckets = E + 1;
+  const int tid = threadIdx.x, wave = tid / kWave;
+  int *cursor = lds + wave * buckets;
+  int *offs = lds + kRouteWaves * buckets;
+  for (int i = tid; i < kRouteWaves * buckets; i += blockDim.x)
+    lds[i] = seg_cursors[(size_t)blockIdx.x * kRouteWaves * buckets + i];
+  for (int b = tid; b <= E; b += blockDim.x) offs[b] = offsets_in[b];
+  __syncthreads();
+  int s = blockIdx.x * kRouteWaves + wave;
+  int seg_begin = min((long long)s * seg, (long long)N), seg_end = min(seg_begin + seg, N);
+  wave_place<I64>(idx, seg_begin, seg_end, E, capacity, cursor, offs, sorted_expert, sorted_idx,
+                  inv_pos);
+}
+
+// ---- work lists ------------------------------------------------------------------------------
+// One wave; experts are walked in order.  Experts with 1..stream_max_rows kept rows go to the
+// streaming list, larger ones are cut into row tiles of kRowTile rows.
+__global__ void build_schedule_kernel(const int *counts, const int *offsets, int N, int E,
+                                      int capacity, int stream_max_rows, int *sched) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  int *row_tiles = sched + kSchedHeader;
+  int *small = row_tiles + 8 * sched_max_row_tiles(N, E);
+  int n_tiles = 0, n_small = 0, n_active = 0, n_kept = 0;
+  for (int e = 0; e < E; ++e) {
+    int kept = min(counts[e], capacity);
+    if (kept <= 0) continue;
+    ++n_active;
+    n_kept += kept;
+    int first = offsets[e];
+    if (kept <= stream_max_rows) {
+      int *s = small + 4 * n_small++;
+      s[0] = e; s[1] = first; s[2] = kept; s[3] = 0;
+    } else {
+      int gfirst = n_tiles, gcount = ceil_div(kept, kRowTile);
+      for (int r = 0; r < kept; r += kRowTile) {
+        int *t = row_tiles + 8 * n_tiles++;
+        t[0] = e; t[1] = first + r; t[2] = min(kRowTile, kept - r); t[3] = gfirst; t[4] = gcount;
+        t[5] = 0; t[6] = 0; t[7] = 0;
+      }
+    }
+  }
+  sched[0] = n_tiles; sched[1] = n_small; sched[2] = n_active; sched[3] = n_kept;
+  sched[4] = 0; sched[5] = 0; sched[6] = 0; sched[7] = 0;
+}
+
+}  // namespace yamoe
+
+using namespace yamoe;
+
+extern "C" size_t yamoe_route_workspace_bytes(int32_t N, int32_t E) {
+  if (N <= kSingleBlockMaxN) return 256;
+  int seg = 2048;
+  int n_seg = ceil_div(ceil_div(N, seg), kRouteWaves) * kRouteWaves;
+  return align_up((size_t)n_seg * (E + 1) * sizeof(int), 256);
+}
+
+extern "C" int yamoe_route(const void *router_indices, int32_t idx_i64, int32_t N, int32_t E,
+                           int32_t capacity, int32_t *sorted_expert, int32_t *sorted_idx,
+                           int32_t *counts, int32_t *offsets, int32_t *inv_pos, void *workspace,
+                           size_t workspace_bytes, void *stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (N < 0 || E <= 0 || E + 1 > kRouteMaxBuckets) {
+    set_error("yamoe_route: need N >= 0 and 1 <= E < %d (got N=%d E=%d)", kRouteMaxBuckets, N, E);
+    return YAMOE_E_ARG;
+  }
+  if (!counts || !offsets || (N > 0 && (!router_indices || !sorted_expert || !sorted_idx || !inv_pos))) {
+    set_error("yamoe_route: null pointer");
+    return YAMOE_E_ARG;
+  }
+  if (capacity < 0) capacity = 0;
+  const int buckets = E + 1;
+  if (N <= kSingleBlockMaxN) {
+    size_t lds = ((size_t)kRouteWaves * buckets + buckets + buckets + 1 + kRouteWaves + 1) * sizeof(int);
+    if (idx_i64)
+      hipLaunchKernelGGL(route_single_kernel<true>, dim3(1), dim3(kRouteThreads), lds, stream,
+                         router_indices, N, E, capacity, sorted_expert, sorted_idx, counts, offsets, inv_pos);
+    else
+      hipLaunchKernelGGL(route_single_kernel<false>, dim3(1), dim3(kRouteThreads), lds, stream,
+                         router_indices, N, E, capacity, sorted_expert, sorted_idx, counts, offsets, inv_pos);
+    return check_launch("route_single_kernel");
+  }
+  if (workspace_bytes < yamoe_route_workspace_bytes(N, E) || !workspace) {
+    set_error("yamoe_route: workspace too small (%zu < %zu)", workspace_bytes, yamoe_route_workspace_bytes(N, E));
+    return YAMOE_E_WORKSPACE;
+  }
+  const int seg = 2048;
+  const int n_blocks = ceil_div(ceil_div(N, seg), kRouteWaves);
+  const int n_seg = n_blocks * kRouteWaves;
+  int *seg_counts = (int *)workspace;
+  size_t lds_a = (size_t)kRouteWaves * buckets * sizeof(int);
+  size_t lds_b = ((size_t)buckets * 2 + 1 + kRouteWaves + 1) * sizeof(int);
+  size_t lds_c = ((size_t)kRouteWaves * buckets + buckets) * sizeof(int);
+  if (idx_i64)
+    hipLaunchKernelGGL(route_hist_kernel<true>, dim3(n_blocks), dim3(kRouteThreads), lds_a, stream,
+                       router_indices, N, E, seg, seg_counts);
+  else
+    hipLaunchKernelGGL(route_hist_kernel<false>, dim3(n_blocks), dim3(kRouteThreads), lds_a, stream,
+                       router_indices, N, E, seg, seg_counts);
+  int rc = check_launch("route_hist_kernel");
+  if (rc) return rc;
+  hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(kRouteThreads), lds_b, stream, seg_counts, n_seg, E,
+                     counts, offsets);
+  rc = check_launch("route_scan_kernel");
+  if (rc) return rc;
+  if (idx_i64)
+    hipLaunchKernelGGL(route_place_kernel<true>, dim3(n_blocks), dim3(kRouteThreads), lds_c, stream,
+                       router_indices, N, E, capacity, seg, seg_counts, offsets, sorted_expert, sorted_idx, inv_pos);
+  else
+    hipLaunchKernelGGL(route_place_kernel<false>, dim3(n_blocks), dim3(kRouteThreads), lds_c, stream,
+                       router_indices, N, E, capacity, seg, seg_counts, offsets, sorted_expert, sorted_idx, inv_pos);
+  return check_launch("route_place_kernel");
+}
+
+extern "C" size_t yamoe_schedule_bytes(int32_t N, int32_t E) {
+  size_t words = kSchedHeader + 8 * (size_t)sched_max_row_tiles(N, E) + 4 * (size_t)sched_max_small(N, E);
+  return align_up(words * sizeof(int), 256);
+}
+
+extern "C" int yamoe_build_schedule(const int32_t *counts, const int32_t *offsets, int32_t N, int32_t E,
+                                    int32_t capacity, int32_t stream_max_rows, void *schedule,
+                                    size_t schedule_bytes, void *stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (!counts || !offsets || !schedule || N < 0 || E <= 0) {
+    set_error("yamoe_build_schedule: bad argument");
+    return YAMOE_E_ARG;
+  }
+  if (schedule_bytes < yamoe_schedule_bytes(N, E)) {
+    set_error("yamoe_build_schedule: schedule region too small");
+    return YAMOE_E_WORKSPACE;
+  }
+  if (capacity < 0) capacity = 0;
+  if (stream_max_rows < 0) stream_max_rows = 0;
+  if (stream_max_rows > kStreamMaxRows) stream_max_rows = kStreamMaxRows;
+  hipLaunchKernelGGL(build_schedule_kernel, dim3(1), dim3(kWave), 0, stream, counts, offsets, N, E, capacity,
+                     stream_max_rows, (int *)schedule);
+  return check_launch("build_schedule_kernel");
+}

@@ -1,0 +1,199 @@
+// Weight-streaming path for experts with at most 16 kept rows (the decode regime).
+//
+// Such an expert does 2*rows flops per weight element, far below the machine balance, so the job
+// is to pull each expert's weights through the chip once at HBM rate.  A workgroup owns one
+// (expert, 128-column slab) of a [K, N] weight matrix.  Its 4 wavefronts take the 32-row k-steps
+// of the slab round-robin; in a step every lane fetches an 8(k) x 8(column) block as eight 16-byte
+// loads (a wave reads 32 rows x 256 contiguous bytes), transposes it in registers and feeds it to
+// eight v_mfma_f32_16x16x32 instructions whose 16-row A operand is the expert's (zero-padded)
+// activations.  No LDS is touched until the final cross-wave reduction.  Two steps of loads are
+// kept in flight per wave, 8 waves per CU.
+//
+// The lane that holds accumulator column c of MFMA j owns output column 8c + j, so the 8
+// accumulators of a lane are 8 consecutive output columns: the interleaved (gate, up) pairs of the
+// clamped SwiGLU (csrc/moe.cpp:164-180) meet in one lane.
+#include "common.h"
+
+namespace yamoe {
+
+constexpr int kStreamThreads = 256;
+constexpr int kStreamWaves = 4;
+constexpr int kSlabCols = 128;
+
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
+template <typename T> struct Mma16;
+template <> struct Mma16<bf16_t> {
+  __device__ static inline f32x4v run(const u32x4 &a, const u32x4 &b, f32x4v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                   0, 0, 0);
+  }
+};
+template <> struct Mma16<f16_t> {
+  __device__ static inline f32x4v run(const u32x4 &a, const u32x4 &b, f32x4v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
+                                                  0, 0);
+  }
+};
+
+struct StreamArgs {
+  const void *A;       // activations [rows, lda], k-contiguous
+  const void *B;       // weights [E, Kd, Nd]
+  const void *bias;    // [E, Nd] or null
+  void *C;             // GLU: act [rows, Nd/2]; else [rows, Nd]
+  void *C2;            // GLU: optional pre-activations [rows, Nd]
+  const int *a_rows;   // optional gather: source row = a_rows[p] / a_div
+  const int *sched;
+  int a_div, Kd, Nd, lda, ldc, n_slabs, N, E;
+};
+
+template <typename T, bool GLU, bool GATHER>
+__global__ __launch_bounds__(kStreamThreads, 2) void stream_gemm_kernel(const StreamArgs args) {
+  __shared__ float red[kStreamWaves * 8 * 4 * kWave];  // [wave][j][v][lane]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const ScheduleView sv = schedule_view(args.sched, args.N, args.E);
+  const int n_small = sv.hdr[1];
+  const int s = blockIdx.x / args.n_slabs;
+  if (s >= n_small) return;
+  const int slab = blockIdx.x - s * args.n_slabs;
+  const int expert = sv.small[4 * s], first = sv.small[4 * s + 1], rows = sv.small[4 * s + 2];
+
+  const int c16 = lane & 15, g = lane >> 4;
+  const int col0 = slab * kSlabCols + c16 * 8;  // first of this lane's 8 output columns
+  const bool col_ok = col0 < args.Nd;
+  const T *Bp = (const T *)args.B + (long long)expert * args.Kd * args.Nd + col0;
+
+  // A operand: row c16 of the expert (zero beyond `rows`), 8 consecutive k starting at 8 g
+  const bool a_ok = c16 < rows;
+  long long a_src = first + (a_ok ? c16 : 0);
+  if (GATHER) a_src = args.a_rows[a_src] / args.a_div;
+  const T *Ap = (const T *)args.A + a_src * args.lda + g * 8;
+
+  f32x4v acc[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) acc[j] = (f32x4v){0.f, 0.f, 0.f, 0.f};
+
+  const int n_steps = (args.Kd + 31) / 32;
+  u32x4 bw0[8], bw1[8], aw0, aw1;
+
+  auto fetch = [&](int step, u32x4 (&bw)[8], u32x4 &aw) {
+    int k0 = step * 32;
+    int ka = k0 + g * 8;
+    aw = (u32x4){0, 0, 0, 0};
+    if (a_ok && ka < args.Kd) aw = *(const u32x4 *)(Ap + k0);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int k = ka + i;
+      u32x4 v = {0, 0, 0, 0};
+      if (col_ok && k < args.Kd) v = __builtin_nontemporal_load((const u32x4 *)(Bp + (long long)k * args.Nd));
+      bw[i] = v;
+    }
+  };
+  auto consume = [&](const u32x4 (&bw)[8], const u32x4 &aw) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+      u32x4 col;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) col[d] = __builtin_amdgcn_perm(bw[2 * d + 1][j >> 1], bw[2 * d][j >> 1], sel);
+      acc[j] = Mma16<T>::run(aw, col, acc[j]);
+    }
+  };
+
+  // steps wave, wave+4, ... ; two in flight
+  int step = wave;
+  if (step < n_steps) fetch(step, bw0, aw0);
+  while (step < n_steps) {
+    if (step + kStreamWaves < n_steps) fetch(step + kStreamWaves, bw1, aw1);
+    consume(bw0, aw0);
+    step += kStreamWaves;
+    if (step >= n_steps) break;
+    if (step + kStreamWaves < n_steps) fetch(step + kStreamWaves, bw0, aw0);
+    consume(bw1, aw1);
+    step += kStreamWaves;
+  }
+
+  // ---- reduce the 4 partial sums and finish -----------------------------------------------------
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) red[((wave * 8 + j) * 4 + v) * kWave + lane] = acc[j][v];
+  __syncthreads();
+
+  // wave w finishes accumulator columns j = 2w, 2w+1 (one gate/up pair per lane)
+  float sum[2][4];
+#pragma unroll
+  for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      float t = 0.f;
+#pragma unroll
+      for (int w = 0; w < kStreamWaves; ++w) t += red[((w * 8 + 2 * wave + jj) * 4 + v) * kWave + lane];
+      sum[jj][v] = t;
+    }
+  const int col = col0 + 2 * wave;
+  if (!col_ok) return;
+  float b0 = 0.f, b1 = 0.f;
+  if (args.bias != nullptr) {
+    const T *bp = (const T *)args.bias + (long long)expert * args.Nd + col;
+    b0 = ElemTraits<T>::to_f32(bp[0]);
+    b1 = ElemTraits<T>::to_f32(bp[1]);
+  }
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    int r = g * 4 + v;
+    if (r >= rows) continue;
+    long long orow = first + r;
+    float x0 = sum[0][v] + b0, x1 = sum[1][v] + b1;
+    if (GLU) {
+      ((T *)args.C)[orow * args.ldc + (col >> 1)] = ElemTraits<T>::from_f32(glu_forward(x0, x1));
+      if (args.C2 != nullptr) {
+        T *P = (T *)args.C2 + orow * args.Nd + col;
+        P[0] = ElemTraits<T>::from_f32(x0);
+        P[1] = ElemTraits<T>::from_f32(x1);
+      }
+    } else {
+      T *O = (T *)args.C + orow * args.ldc + col;
+      O[0] = ElemTraits<T>::from_f32(x0);
+      O[1] = ElemTraits<T>::from_f32(x1);
+    }
+  }
+}
+
+template <typename T, bool GLU, bool GATHER>
+static int launch_stream(const StreamArgs &a, hipStream_t stream) {
+  long long blocks = (long long)sched_max_small(a.N, a.E) * a.n_slabs;
+  if (blocks <= 0) return 0;
+  hipLaunchKernelGGL((stream_gemm_kernel<T, GLU, GATHER>), dim3((unsigned)blocks), dim3(kStreamThreads), 0, stream, a);
+  return check_launch("stream_gemm_kernel");
+}
+
+template <typename T>
+int stream_gate_up(const void *x, const int *sorted_idx, const void *w, const void *bias, void *act, void *pre,
+                   const void *sched, int N, int K, int E, int H, int I, hipStream_t stream) {
+  StreamArgs a = {};
+  a.A = x; a.B = w; a.bias = bias; a.C = act; a.C2 = pre; a.a_rows = sorted_idx; a.a_div = K;
+  a.sched = (const int *)sched; a.Kd = H; a.Nd = 2 * I; a.lda = H; a.ldc = I;
+  a.n_slabs = ceil_div(2 * I, kSlabCols); a.N = N; a.E = E;
+  return launch_stream<T, true, true>(a, stream);
+}
+
+template <typename T>
+int stream_down(const void *act, const void *w, const void *bias, void *y, const void *sched, int N, int E, int H,
+                int I, hipStream_t stream) {
+  StreamArgs a = {};
+  a.A = act; a.B = w; a.bias = bias; a.C = y; a.sched = (const int *)sched;
+  a.Kd = I; a.Nd = H; a.lda = I; a.ldc = H;
+  a.n_slabs = ceil_div(H, kSlabCols); a.N = N; a.E = E;
+  return launch_stream<T, false, false>(a, stream);
+}
+
+#define YAMOE_INSTANTIATE_STREAM(T)                                                                                  \
+  template int stream_gate_up<T>(const void *, const int *, const void *, const void *, void *, void *, const void *, \
+                                 int, int, int, int, int, hipStream_t);                                              \
+  template int stream_down<T>(const void *, const void *, const void *, void *, const void *, int, int, int, int,    \
+                              hipStream_t);
+YAMOE_INSTANTIATE_STREAM(bf16_t)
+YAMOE_INSTANTIATE_STREAM(f16_t)
+
+}  // namespace yamoe

@@ -1,0 +1,187 @@
+// Torch operator layer over the C ABI of libyamoe_hip.so.
+//
+// Registers `experts` and `experts_backward` with the schemas of drbh/yamoe
+// (torch-ext/torch_binding.cpp:58-83) for the GPU dispatch key (which torch-ROCm spells CUDA).
+// This file is host-only C++: it checks arguments the way experts_cuda does
+// (csrc/moe.cpp:58-96), allocates the output and one workspace tensor from torch's caching
+// allocator, and hands raw pointers plus the current HIP stream to the library.  No host
+// synchronisation, no `.item()`, so the ops can be captured in a HIP graph.
+#include <ATen/ATen.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <torch/library.h>
+
+#include <vector>
+
+#include "yamoe_hip.h"
+
+namespace {
+
+int dtype_code(const at::Tensor &t, const char *name) {
+  switch (t.scalar_type()) {
+    case at::kFloat: return YAMOE_F32;
+    case at::kHalf: return YAMOE_F16;
+    case at::kBFloat16: return YAMOE_BF16;
+    default:
+      TORCH_CHECK(false, name, " must be float32, float16 or bfloat16, got ", t.scalar_type());
+  }
+  return -1;
+}
+
+void check_rc(int rc, const char *what) {
+  TORCH_CHECK(rc == 0, what, " failed (", rc, "): ", yamoe_last_error());
+}
+
+struct Checked {
+  yamoe_problem p;
+  at::Tensor hidden, idx, rw, wgu, bgu, wd, bd;
+};
+
+Checked check_inputs(const at::Tensor &hidden_states, const at::Tensor &router_indices,
+                     const at::Tensor &routing_weights, const at::Tensor &gate_up_proj,
+                     const at::Tensor &gate_up_proj_bias, const at::Tensor &down_proj,
+                     const at::Tensor &down_proj_bias, int64_t expert_capacity, int64_t num_experts, int64_t top_k) {
+  TORCH_CHECK(hidden_states.is_cuda(), "hidden_states must be on the GPU");
+  TORCH_CHECK(router_indices.is_cuda(), "router_indices must be on the GPU");
+  TORCH_CHECK(routing_weights.is_cuda(), "routing_weights must be on the GPU");
+  TORCH_CHECK(gate_up_proj.is_cuda(), "gate_up_proj must be on the GPU");
+  TORCH_CHECK(gate_up_proj_bias.is_cuda(), "gate_up_proj_bias must be on the GPU");
+  TORCH_CHECK(down_proj.is_cuda(), "down_proj must be on the GPU");
+  TORCH_CHECK(down_proj_bias.is_cuda(), "down_proj_bias must be on the GPU");
+
+  TORCH_CHECK(hidden_states.dim() == 2, "hidden_states must be 2D [T, H]");
+  TORCH_CHECK(router_indices.dim() == 2, "router_indices must be 2D [T, K]");
+  TORCH_CHECK(routing_weights.dim() == 2, "routing_weights must be 2D [T, E] or [T, K]");
+  TORCH_CHECK(gate_up_proj.dim() == 3, "gate_up_proj must be 3D [E, H, 2*I]");
+  TORCH_CHECK(gate_up_proj_bias.dim() == 2, "gate_up_proj_bias must be 2D [E, 2*I]");
+  TORCH_CHECK(down_proj.dim() == 3, "down_proj must be 3D [E, I, H]");
+  TORCH_CHECK(down_proj_bias.dim() == 2, "down_proj_bias must be 2D [E, H]");
+
+  const int64_t T = hidden_states.size(0), H = hidden_states.size(1), E = num_experts, K = top_k;
+  TORCH_CHECK(E > 0 && K > 0, "num_experts and top_k must be positive");
+  TORCH_CHECK(router_indices.size(0) == T && router_indices.size(1) == K, "router_indices must be [T, K]");
+  TORCH_CHECK(routing_weights.size(0) == T && (routing_weights.size(1) == K || routing_weights.size(1) == E),
+              "routing_weights must be [T, K] or [T, E]");
+  TORCH_CHECK(gate_up_proj.size(0) == E && gate_up_proj.size(1) == H && gate_up_proj.size(2) % 2 == 0,
+              "gate_up_proj must be [E, H, 2*I]");
+  const int64_t I = gate_up_proj.size(2) / 2;
+  TORCH_CHECK(gate_up_proj_bias.size(0) == E && gate_up_proj_bias.size(1) == 2 * I,
+              "gate_up_proj_bias must be [E, 2*I]");
+  TORCH_CHECK(down_proj.size(0) == E && down_proj.size(1) == I && down_proj.size(2) == H,
+              "down_proj must be [E, I, H]");
+  TORCH_CHECK(down_proj_bias.size(0) == E && down_proj_bias.size(1) == H, "down_proj_bias must be [E, H]");
+  TORCH_CHECK(router_indices.scalar_type() == at::kLong || router_indices.scalar_type() == at::kInt,
+              "router_indices must be int64 or int32");
+  const auto dt = hidden_states.scalar_type();
+  TORCH_CHECK(routing_weights.scalar_type() == dt && gate_up_proj.scalar_type() == dt &&
+                  gate_up_proj_bias.scalar_type() == dt && down_proj.scalar_type() == dt &&
+                  down_proj_bias.scalar_type() == dt,
+              "all floating tensors must share hidden_states' dtype");
+  const auto dev = hidden_states.device();
+  TORCH_CHECK(router_indices.device() == dev && routing_weights.device() == dev && gate_up_proj.device() == dev &&
+                  gate_up_proj_bias.device() == dev && down_proj.device() == dev && down_proj_bias.device() == dev,
+              "all tensors must be on the same device");
+  TORCH_CHECK(T * K <= (int64_t)1 << 30, "T*K too large");
+
+  Checked c;
+  c.hidden = hidden_states.contiguous();
+  c.idx = router_indices.contiguous();
+  c.rw = routing_weights.contiguous();
+  c.wgu = gate_up_proj.contiguous();
+  c.bgu = gate_up_proj_bias.contiguous();
+  c.wd = down_proj.contiguous();
+  c.bd = down_proj_bias.contiguous();
+  c.p.T = (int32_t)T;
+  c.p.K = (int32_t)K;
+  c.p.E = (int32_t)E;
+  c.p.H = (int32_t)H;
+  c.p.I = (int32_t)I;
+  c.p.capacity = (int32_t)std::min<int64_t>(std::max<int64_t>(expert_capacity, 0), INT32_MAX);
+  c.p.dtype = dtype_code(hidden_states, "hidden_states");
+  c.p.idx_i64 = router_indices.scalar_type() == at::kLong ? 1 : 0;
+  c.p.rw_cols = (int32_t)routing_weights.size(1);
+  return c;
+}
+
+at::Tensor experts(at::Tensor hidden_states, at::Tensor router_indices, at::Tensor routing_weights,
+                   at::Tensor gate_up_proj, at::Tensor gate_up_proj_bias, at::Tensor down_proj,
+                   at::Tensor down_proj_bias, int64_t expert_capacity, int64_t num_experts, int64_t top_k) {
+  Checked c = check_inputs(hidden_states, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
+                           down_proj_bias, expert_capacity, num_experts, top_k);
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(c.hidden.device());
+  at::Tensor out = at::empty_like(c.hidden);
+  if (c.p.T == 0) return out;
+  size_t ws_bytes = yamoe_experts_workspace_bytes(&c.p);
+  TORCH_CHECK(ws_bytes > 0, "experts: ", yamoe_last_error());
+  at::Tensor ws = at::empty({(int64_t)ws_bytes}, c.hidden.options().dtype(at::kByte));
+  void *stream = (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+  check_rc(yamoe_experts_forward(&c.p, c.hidden.data_ptr(), c.idx.data_ptr(), c.rw.data_ptr(), c.wgu.data_ptr(),
+                                 c.bgu.data_ptr(), c.wd.data_ptr(), c.bd.data_ptr(), out.data_ptr(), ws.data_ptr(),
+                                 ws_bytes, stream),
+           "yamoe_experts_forward");
+  return out;
+}
+
+std::vector<at::Tensor> experts_backward(const at::Tensor &grad_out, const at::Tensor &hidden_states,
+                                         const at::Tensor &router_indices, const at::Tensor &routing_weights,
+                                         const at::Tensor &gate_up_proj, const at::Tensor &gate_up_proj_bias,
+                                         const at::Tensor &down_proj, const at::Tensor &down_proj_bias,
+                                         int64_t expert_capacity, int64_t num_experts, int64_t top_k) {
+  TORCH_CHECK(grad_out.is_cuda(), "grad_out must be on the GPU");
+  Checked c = check_inputs(hidden_states, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
+                           down_proj_bias, expert_capacity, num_experts, top_k);
+  const int64_t T = c.p.T, H = c.p.H, K = c.p.K;
+  TORCH_CHECK(grad_out.scalar_type() == c.hidden.scalar_type(), "grad_out must share hidden_states' dtype");
+  TORCH_CHECK(grad_out.numel() == T * H || grad_out.numel() == T * K * H, "grad_out numel must be T*H or T*K*H");
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(c.hidden.device());
+  // a [T,K,H] gradient is first summed over the slot axis (csrc/experts_backward.cu:224-228)
+  at::Tensor gy = grad_out.numel() == T * H ? grad_out.contiguous().view({T, H})
+                                            : grad_out.contiguous().view({T, K, H}).sum(1).contiguous();
+  at::Tensor d_hidden = at::empty_like(c.hidden);
+  at::Tensor d_routing = at::empty_like(c.rw);
+  at::Tensor d_wgu = at::empty_like(c.wgu);
+  at::Tensor d_bgu = at::empty_like(c.bgu);
+  at::Tensor d_wd = at::empty_like(c.wd);
+  at::Tensor d_bd = at::empty_like(c.bd);
+  size_t ws_bytes = yamoe_experts_backward_workspace_bytes(&c.p);
+  TORCH_CHECK(ws_bytes > 0, "experts_backward: ", yamoe_last_error());
+  at::Tensor ws = at::empty({(int64_t)ws_bytes}, c.hidden.options().dtype(at::kByte));
+  void *stream = (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+  check_rc(yamoe_experts_backward(&c.p, gy.data_ptr(), c.hidden.data_ptr(), c.idx.data_ptr(), c.rw.data_ptr(),
+                                  c.wgu.data_ptr(), c.bgu.data_ptr(), c.wd.data_ptr(), c.bd.data_ptr(),
+                                  d_hidden.data_ptr(), d_routing.data_ptr(), d_wgu.data_ptr(), d_bgu.data_ptr(),
+                                  d_wd.data_ptr(), d_bd.data_ptr(), ws.data_ptr(), ws_bytes, stream),
+           "yamoe_experts_backward");
+  return {d_hidden, d_routing, d_wgu, d_bgu, d_wd, d_bd};
+}
+
+}  // namespace
+
+TORCH_LIBRARY(_yamoe_amd_ops, ops) {
+  ops.def("experts("
+          "Tensor hidden_states, "
+          "Tensor router_indices, "
+          "Tensor routing_weights, "
+          "Tensor gate_up_proj, "
+          "Tensor gate_up_proj_bias, "
+          "Tensor down_proj, "
+          "Tensor down_proj_bias, "
+          "int expert_capacity, "
+          "int num_experts, "
+          "int top_k) -> Tensor");
+  ops.impl("experts", c10::DispatchKey::CUDA, &experts);
+
+  ops.def("experts_backward("
+          "Tensor grad_out, "
+          "Tensor hidden_states, "
+          "Tensor router_indices, "
+          "Tensor routing_weights, "
+          "Tensor gate_up_proj, "
+          "Tensor gate_up_proj_bias, "
+          "Tensor down_proj, "
+          "Tensor down_proj_bias, "
+          "int expert_capacity, "
+          "int num_experts, "
+          "int top_k) -> Tensor[]");
+  ops.impl("experts_backward", c10::DispatchKey::CUDA, &experts_backward);
+}

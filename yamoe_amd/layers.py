@@ -1,0 +1,72 @@
+"""Autograd glue for the `experts` op, mirroring `_ExpertsFn` of drbh/yamoe
+(torch-ext/yamoe/layers.py:6-100): same saved tensors, same order and arity of returned gradients.
+"""
+import torch
+
+from ._ops import ops
+
+
+class _ExpertsFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, hidden_flat, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
+                down_proj_bias, expert_capacity, num_experts, top_k, enable_router_grads):
+        out = ops.experts(hidden_flat, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
+                          down_proj_bias, expert_capacity, num_experts, top_k)
+        ctx.expert_capacity = expert_capacity
+        ctx.num_experts = num_experts
+        ctx.top_k = top_k
+        ctx.enable_router_grads = bool(enable_router_grads)
+        ctx.save_for_backward(hidden_flat, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias,
+                              down_proj, down_proj_bias)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        saved = ctx.saved_tensors
+        d_hidden, d_routing, d_wgu, d_bgu, d_wd, d_bd = ops.experts_backward(
+            grad_output.contiguous(), *saved, ctx.expert_capacity, ctx.num_experts, ctx.top_k)
+        if not ctx.enable_router_grads:
+            d_routing = None
+        return d_hidden, None, d_routing, d_wgu, d_bgu, d_wd, d_bd, None, None, None, None
+
+
+def experts_autograd(hidden_flat, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
+                     down_proj_bias, expert_capacity, num_experts, top_k, enable_router_grads=True):
+    """Differentiable `experts`: gradients flow to hidden states, weights, biases and (optionally)
+    the routing weights."""
+    return _ExpertsFn.apply(hidden_flat, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
+                            down_proj_bias, expert_capacity, num_experts, top_k, enable_router_grads)
+
+
+class Yamoe(torch.nn.Module):
+    """Drop-in `forward` for a GPT-OSS MLP block (router + experts), the role of `Yamoe.forward` in
+    drbh/yamoe (torch-ext/yamoe/layers.py:106-218).  The host module provides `self.router`
+    (weight [E,H], bias [E]) and `self.experts` (gate_up_proj, gate_up_proj_bias, down_proj,
+    down_proj_bias).  Unlike the reference, no assignment is dropped (capacity = tokens) and the
+    router gradient is kept when `enable_router_grads` is set.
+    """
+
+    can_torch_compile: bool = False
+
+    def forward(self, hidden_states):
+        batch, seq, hidden = hidden_states.shape
+        num_experts = getattr(self, "num_experts", 32)
+        top_k = getattr(self, "top_k", 4)
+        x_flat = hidden_states.reshape(-1, hidden)
+        logits = torch.nn.functional.linear(x_flat, self.router.weight, self.router.bias)
+        top_vals, router_indices = torch.topk(logits, top_k, dim=-1)
+        top_w = torch.nn.functional.softmax(top_vals, dim=-1, dtype=top_vals.dtype)
+        router_scores = torch.zeros_like(logits).scatter_(1, router_indices, top_w)
+        I = self.experts.down_proj.shape[1]
+        gate_up = self.experts.gate_up_proj[:, :, : 2 * I].contiguous()
+        gate_up_bias = self.experts.gate_up_proj_bias[:, : 2 * I].contiguous()
+        capacity = x_flat.shape[0]
+        if torch.is_grad_enabled() and getattr(self, "enable_router_grads", False):
+            out = experts_autograd(x_flat, router_indices, router_scores, gate_up, gate_up_bias,
+                                   self.experts.down_proj, self.experts.down_proj_bias, capacity, num_experts, top_k,
+                                   True)
+        else:
+            with torch.no_grad():
+                out = ops.experts(x_flat, router_indices, router_scores, gate_up, gate_up_bias,
+                                  self.experts.down_proj, self.experts.down_proj_bias, capacity, num_experts, top_k)
+        return out.view(batch, seq, hidden), router_scores
