@@ -1,0 +1,198 @@
+#!/usr/bin/env python3
+"""Benchmark of the expert-layer forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one `experts()` forward (torch op -> C ABI -> HIP kernels) over one synthetic batch of the
+GPT-OSS-20B shaped layer: 4096 tokens, hidden = intermediate = 2880, 32 experts, top-4, bf16, inputs
+already resident in HBM.  Prints ONE JSON line.  `value` is algorithmic TFLOP/s of the whole op
+(6*H*I flop per kept (token, expert) assignment divided by the step time).
+
+Also on the line:
+  roofline      the dominant kernel (the gate_up grouped GEMM), timed on its own with HIP events on
+                the stream it runs on: algorithmic flop per launch / average launch time vs the
+                2.5 PFLOP/s dense bf16 MFMA peak
+  decode        the 64-token / 128-expert decode workload: algorithmic HBM bytes per step / step time
+                vs the 8 TB/s HBM peak
+  cpu_baseline  the CPU oracle (oracle/yamoe_oracle.py, the loop-over-experts path the reference itself
+                takes on a CPU) timed on this box's host cores on a slice of the same batch
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+# HBM bytes per launch of the gate_up GEMM from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (see the
+# counter summary under profiles/); None until measured.
+GATE_UP_TRAFFIC_BYTES = None
+
+
+def event_time_ms(fn, iters):
+    import torch
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / iters
+
+
+def device_weights(E, H, I, dtype, std, seed, device):
+    """Weights drawn on the device (N(0, std)); used where drawing on the host would take minutes."""
+    import torch
+    g = torch.Generator(device=device).manual_seed(seed)
+
+    def draw(shape):
+        t = torch.empty(shape, dtype=dtype, device=device)
+        for e in range(shape[0]):
+            t[e] = (torch.randn(shape[1:], generator=g, device=device) * std).to(dtype)
+        return t
+    return dict(gate_up_proj=draw((E, H, 2 * I)), gate_up_proj_bias=draw((E, 2 * I)), down_proj=draw((E, I, H)),
+                down_proj_bias=draw((E, H)))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-decode", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus %d is not supported (the expert layer here is the "
+              "single-GPU share of an expert-parallel layout)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import yamoe_amd
+    from yamoe_amd import _cabi, workloads
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    # ---------------- GPT-OSS-20B shaped layer ----------------------------------------------------------
+    cfg = workloads.CONFIGS["gptoss20b"]
+    T, H, I, E, K = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["K"]
+    host, _ = workloads.make_config("gptoss20b", seed=0, weights=False)
+    d = {k: v.to(dev) for k, v in host.items()}
+    d.update(device_weights(E, H, I, torch.bfloat16, cfg["w_std"], 1, dev))
+    order = ("hidden", "router_indices", "routing_weights", "gate_up_proj", "gate_up_proj_bias", "down_proj",
+             "down_proj_bias")
+    a = [d[k] for k in order]
+    n_rows = T * K  # capacity = T keeps every assignment
+    flop = n_rows * workloads.FWD_FLOP_PER_ROW(H, I)
+
+    def step():
+        return yamoe_amd.experts(*a, T, E, K)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev_ms = event_time_ms(step, args.steps)
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = max(ev_ms, wall_ms)
+    value = flop / (ms_per_step * 1e-3) / 1e12
+
+    # ---------------- dominant kernel on its own: gate_up grouped GEMM -----------------------------------
+    se, si, counts, offsets, inv = _cabi.route(d["router_indices"], E, T)
+    sched = _cabi.build_schedule(counts, offsets, n_rows, T, 16)
+    act = _cabi.gate_up(d["hidden"], si, d["gate_up_proj"], d["gate_up_proj_bias"], sched, K)
+    gu_ms = event_time_ms(lambda: _cabi.lib().yamoe_gate_up(
+        _cabi._p(d["hidden"]), _cabi._p(si), _cabi._p(d["gate_up_proj"]), _cabi._p(d["gate_up_proj_bias"]),
+        _cabi._p(act), None, _cabi._p(sched), n_rows, K, E, H, I, _cabi.BF16, _cabi._stream()), args.steps)
+    y = _cabi.down(act, d["down_proj"], d["down_proj_bias"], sched)
+    dn_ms = event_time_ms(lambda: _cabi.lib().yamoe_down(
+        _cabi._p(act), _cabi._p(d["down_proj"]), _cabi._p(d["down_proj_bias"]), _cabi._p(y), _cabi._p(sched), n_rows,
+        E, H, I, _cabi.BF16, _cabi._stream()), args.steps)
+    gu_flop = n_rows * 4 * H * I
+    gu_tflops = gu_flop / (gu_ms * 1e-3) / 1e12
+    dn_tflops = n_rows * 2 * H * I / (dn_ms * 1e-3) / 1e12
+    roofline = dict(bound="mfma", kernel="grouped_gemm_kernel<bf16, gate_up + GLU>", achieved=round(gu_tflops, 2),
+                    peak=PEAK_BF16_TFLOPS, unit="TFLOP/s", frac=round(gu_tflops / PEAK_BF16_TFLOPS, 4),
+                    traffic=GATE_UP_TRAFFIC_BYTES, avg_launch_ms=round(gu_ms, 4),
+                    down_gemm=dict(achieved=round(dn_tflops, 2), frac=round(dn_tflops / PEAK_BF16_TFLOPS, 4),
+                                   avg_launch_ms=round(dn_ms, 4)))
+
+    # ---------------- CPU baseline on a slice of the same batch ------------------------------------------
+    cpu_baseline = None
+    parity = None
+    if not args.no_cpu_baseline:
+        from oracle import yamoe_oracle as O
+        sample_tokens = 2048
+        torch.set_num_threads(min(os.cpu_count() or 1, 16))
+        # inputs are converted to the fp32 compute type once, outside the timed region
+        hs = {k: d[k][:sample_tokens].cpu() if k in ("hidden", "router_indices", "routing_weights") else d[k].cpu()
+              for k in order}
+        hs = {k: (v.float() if v.is_floating_point() else v) for k, v in hs.items()}
+        hargs = [hs[k] for k in order]
+        O.experts_loop(*[t[:64] if i < 3 else t for i, t in enumerate(hargs)], compute_dtype=torch.float32)  # warm-up
+        times = []
+        for _ in range(3):
+            t1 = time.perf_counter()
+            ref = O.experts_loop(*hargs, compute_dtype=torch.float32)
+            times.append(time.perf_counter() - t1)
+        cpu_s = sorted(times)[1]
+        cpu_flop = sample_tokens * K * workloads.FWD_FLOP_PER_ROW(H, I)
+        cpu_baseline = dict(value=round(cpu_flop / cpu_s / 1e12, 4), unit="TFLOP/s", cores=torch.get_num_threads(),
+                            kind="port", sample="first %d of the %d tokens of the same batch, fp32 compute on the "
+                            "bf16 inputs, median of 3 runs (%.2f s each)" % (sample_tokens, T, cpu_s))
+        got = step()[:sample_tokens].float().cpu()
+        parity = dict(rel_l2=float("%.3e" % O.rel_l2(got, ref)), max_abs=float("%.3e" % O.max_abs(got, ref)),
+                      tolerance=1e-2, against="fp32 oracle on the first %d tokens" % sample_tokens)
+        del hs, hargs
+
+    # ---------------- decode workload: 64 tokens, 128 experts ---------------------------------------------
+    decode = None
+    if not args.no_decode:
+        del d, a, act, y
+        torch.cuda.empty_cache()
+        dc = workloads.CONFIGS["decode"]
+        Td, Ed, Kd = dc["T"], dc["E"], dc["K"]
+        hostd, _ = workloads.make_config("decode", seed=0, weights=False)
+        dd = {k: v.to(dev) for k, v in hostd.items()}
+        dd.update(device_weights(Ed, H, I, torch.bfloat16, dc["w_std"], 2, dev))
+        ad = [dd[k] for k in order]
+        n_active = int((np.bincount(hostd["router_indices"].numpy().ravel(), minlength=Ed) > 0).sum())
+        nbytes = workloads.algorithmic_bytes_decode(n_active, Td, Kd, Ed, H, I)
+
+        def dstep():
+            return yamoe_amd.experts(*ad, Td, Ed, Kd)
+
+        for _ in range(args.warmup):
+            dstep()
+        d_ms = event_time_ms(dstep, args.steps)
+        gbs = nbytes / (d_ms * 1e-3) / 1e9
+        decode = dict(metric="experts_fwd_decode_hbm_gbs", value=round(gbs, 1), unit="GB/s", ms_per_step=round(d_ms, 4),
+                      frac_of_hbm_peak=round(gbs / PEAK_HBM_GBS, 4), peak=PEAK_HBM_GBS, active_experts=n_active,
+                      algorithmic_bytes=nbytes,
+                      config=dict(workload="decode: T=64 H=I=2880 E=128 top-4 bf16", tokens=Td, experts=Ed, top_k=Kd))
+
+    line = dict(metric="experts_fwd_tflops", value=round(value, 2), unit="TFLOP/s", n_gpus=1, steps=args.steps,
+                warmup=args.warmup, ms_per_step=round(ms_per_step, 4), higher_is_better=True, scaling="weak",
+                vs_baseline=None, dtype="bf16", data="synthetic",
+                config=dict(workload="gptoss20b: T=4096 H=I=2880 E=32 top-4 bf16, clamped SwiGLU, capacity=T",
+                            tokens=T, hidden=H, intermediate=I, experts=E, top_k=K,
+                            algorithmic_flop=flop),
+                frac_of_mfma_peak=round(value / PEAK_BF16_TFLOPS, 4), roofline=roofline, cpu_baseline=cpu_baseline,
+                parity=parity, decode=decode)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,96 @@
+"""experts_backward through the torch op against autograd through the CPU oracle."""
+import pytest
+import torch
+
+from oracle import yamoe_oracle as O
+from tests.util import args, to_dev
+from yamoe_amd.workloads import make_config, make_inputs
+
+pytestmark = pytest.mark.gpu
+
+NAMES = ("d_hidden", "d_routing", "d_gate_up_proj", "d_gate_up_proj_bias", "d_down_proj", "d_down_proj_bias")
+TOL = {torch.float32: 2e-5, torch.bfloat16: 1e-2, torch.float16: 1e-2}
+
+
+def run_bwd(d, gy, capacity, gpu):
+    import yamoe_amd
+    g = to_dev(d, gpu)
+    E, K = d["gate_up_proj"].shape[0], d["router_indices"].shape[1]
+    grads = yamoe_amd.experts_backward(gy.to(gpu), *args(g), capacity, E, K)
+    torch.cuda.synchronize()
+    return [t.cpu() for t in grads]
+
+
+def check(grads, want, dtype, label):
+    for n, a, b in zip(NAMES, grads, want):
+        assert a.shape == b.shape, (n, a.shape, b.shape)
+        r, m = O.rel_l2(a, b), O.max_abs(a, b)
+        print("%s %s: rel_l2=%.3e max_abs=%.3e" % (label, n, r, m), flush=True)
+        assert r < TOL[dtype], (n, r)
+
+
+SMALL = [
+    (40, 64, 64, 4, 2),       # few rows per expert
+    (700, 64, 96, 3, 2),      # > 256 rows per expert, I != H
+    (513, 264, 136, 5, 3),    # ragged everything
+    (300, 520, 64, 16, 2),    # some empty experts (zipf)
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,H,I,E,K", SMALL)
+def test_backward_small(gpu, dtype, T, H, I, E, K):
+    print("backward_small", dtype, T, H, I, E, K, flush=True)
+    d = make_inputs(T, H, I, E, K, dtype, seed=T, w_std=0.05, bias_std=0.1, zipf=1.5 if E >= 16 else 0.0)
+    gy = torch.randn(T, H, generator=torch.Generator().manual_seed(2)).to(dtype)
+    grads = run_bwd(d, gy, T, gpu)
+    want = O.experts_backward(gy, *args(d), T, compute_dtype=torch.float64 if dtype == torch.float32 else torch.float32)
+    check(grads, want, dtype, "small")
+
+
+@pytest.mark.parametrize("slot_weights", [False, True])
+def test_backward_capacity_and_layouts(gpu, slot_weights):
+    dtype = torch.float32
+    T, H, I, E, K = 200, 64, 64, 4, 2
+    d = make_inputs(T, H, I, E, K, dtype, seed=5, w_std=0.05, bias_std=0.1, zipf=1.0)
+    if slot_weights:
+        d["routing_weights"] = torch.gather(d["routing_weights"], 1, d["router_indices"])
+    gy = torch.randn(T, H, generator=torch.Generator().manual_seed(3))
+    for C in (30, 0):
+        grads = run_bwd(d, gy, C, gpu)
+        want = O.experts_backward(gy, *args(d), C, compute_dtype=torch.float64)
+        if C == 0:
+            assert all(torch.all(g == 0) for g in grads)
+        else:
+            check(grads, want, dtype, "cap%d" % C)
+    # the routing gradient is zero outside the selected experts
+    if not slot_weights:
+        d_rw = run_bwd(d, gy, T, gpu)[1]
+        sel = torch.zeros_like(d_rw, dtype=torch.bool).scatter_(1, d["router_indices"], True)
+        assert torch.all(d_rw[~sel] == 0)
+
+
+def test_autograd_function_matches_op(gpu):
+    """_ExpertsFn wires the six gradients to the right inputs (torch-ext/yamoe/layers.py:50-100)."""
+    import yamoe_amd
+    T, H, I, E, K = 64, 64, 64, 4, 2
+    d = to_dev(make_inputs(T, H, I, E, K, torch.float32, seed=9, w_std=0.05, bias_std=0.1), gpu)
+    leaves = {k: d[k].clone().requires_grad_(True) for k in
+              ("hidden", "routing_weights", "gate_up_proj", "gate_up_proj_bias", "down_proj", "down_proj_bias")}
+    out = yamoe_amd.experts_autograd(leaves["hidden"], d["router_indices"], leaves["routing_weights"],
+                                     leaves["gate_up_proj"], leaves["gate_up_proj_bias"], leaves["down_proj"],
+                                     leaves["down_proj_bias"], T, E, K, True)
+    gy = torch.randn_like(out)
+    out.backward(gy)
+    direct = yamoe_amd.experts_backward(gy, *args(d), T, E, K)
+    for (k, leaf), g in zip(leaves.items(), direct):
+        assert torch.equal(leaf.grad, g), k
+
+
+def test_backward_gptoss20b_full(gpu):
+    """Backward at the GPT-OSS-20B shape, bf16, against fp32 autograd through the oracle."""
+    d, c = make_config("gptoss20b", seed=0)
+    gy = torch.randn(c["T"], c["H"], generator=torch.Generator().manual_seed(4)).to(torch.bfloat16)
+    grads = run_bwd(d, gy, c["T"], gpu)
+    want = O.experts_backward(gy, *args(d), c["T"], compute_dtype=torch.float32)
+    check(grads, want, torch.bfloat16, "gptoss20b")
