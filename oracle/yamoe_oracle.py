@@ -171,6 +171,8 @@ def experts_backward(grad_out, hidden, router_indices, routing_weights, gate_up_
               for t in (hidden, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj, down_proj_bias)]
     out = experts_capacity(leaves[0], router_indices, leaves[1], leaves[2], leaves[3], leaves[4], leaves[5],
                            capacity, compute_dtype)
+    if not out.requires_grad:  # nothing kept (capacity 0 or no tokens): every gradient is zero
+        return tuple(torch.zeros_like(l) for l in leaves)
     grads = torch.autograd.grad(out, leaves, grad_out.reshape(out.shape).to(compute_dtype), allow_unused=True)
     return tuple(torch.zeros_like(l) if g is None else g for g, l in zip(grads, leaves))
 

@@ -125,7 +125,8 @@ static size_t carve_forward(const yamoe_problem *p, void *ws, ForwardBuffers *b)
   b->route_ws_bytes = yamoe_route_workspace_bytes((int)N, p->E);
   b->route_ws = c.take(b->route_ws_bytes);
   b->act = c.take(N * p->I * es);
-  b->y_perm = c.take(N * p->H * es);
+  // sized for the larger of H and I: the backward reuses this region for d_act [N, I]
+  b->y_perm = c.take(N * (size_t)(p->H > p->I ? p->H : p->I) * es);
   return c.used;
 }
 
@@ -142,7 +143,7 @@ static size_t carve_backward(const yamoe_problem *p, void *ws, BackwardBuffers *
   b->pre = c.take(N * 2 * p->I * es);
   b->g_y_perm = c.take(N * p->H * es);
   b->d_pre = c.take(N * 2 * p->I * es);
-  // d_act reuses y_perm (dead after the combine backward); d_x_perm reuses g_y_perm's successor slot
+  // d_act [N, I] reuses the y_perm region (dead after the combine backward)
   b->d_act = b->f.y_perm;
   b->d_x_perm = c.take(N * p->H * es);
   return used + c.used;
