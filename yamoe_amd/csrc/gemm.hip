@@ -27,6 +27,8 @@
 //
 // Replaces batch_mm / torch::bmm on padded [E,C,*] buffers (csrc/batch_mm.cu:7-31) and the ATen
 // bias + clamped-SwiGLU chain (csrc/moe.cpp:161-187; backward csrc/experts_backward.cu:277-311).
+#include <type_traits>
+
 #include "common.h"
 
 namespace yamoe {
@@ -119,25 +121,34 @@ template <> struct BlockTranspose<4> {
 
 // ---- operand loaders -----------------------------------------------------------------------------
 // A "tile operand" is 256 rows x one K slab.  fetch() pulls the slab into 8 x 16-byte registers,
-// commit() writes them to LDS.
+// commit() writes them to LDS.  Loads are unconditional at clamped addresses (rows or columns past
+// the valid range re-read a valid one; their products are never stored), so the main loop has no
+// divergent control flow.  Only the last slab of the contraction can run past k_len; it is fetched
+// with TAIL = true, which zero-fills by select.
 
 // k-contiguous rows: thread -> chunk (tid & 7) of rows (tid >> 3) + 32 i.
 template <typename T>
 struct KContigLoader {
   static constexpr int V = ElemTraits<T>::kVec;
-  const T *base;
-  long long row_off[8];  // element offset of each of this thread's rows
+  const char *base;     // wave-uniform
+  uint32_t row_off[8];  // byte offset of each of this thread's rows (chunk included) from base
   int chunk, Kd;
   u32x4 regs[8];
 
+  template <bool TAIL>
   __device__ inline void fetch(int k0) {
-    int k = k0 + chunk * V;
-    bool ok = k < Kd;
+    const char *slab = base + (long long)k0 * (long long)sizeof(T);
+    if (!TAIL) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      u32x4 v = {0, 0, 0, 0};
-      if (ok) v = *(const u32x4 *)(base + row_off[i] + k);
-      regs[i] = v;
+      for (int i = 0; i < 8; ++i) regs[i] = *(const u32x4 *)(slab + row_off[i]);
+    } else {
+      const bool ok = k0 + chunk * V < Kd;
+      if (!ok) slab = base;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        u32x4 v = *(const u32x4 *)(slab + row_off[i]);
+        regs[i] = ok ? v : (u32x4){0, 0, 0, 0};
+      }
     }
   }
   __device__ inline void commit(char *lds, int tid) {
@@ -151,26 +162,44 @@ struct KContigLoader {
 
 // Operand stored as [k][row] with `row` contiguous: element (k, r) at base + k * ld + r.
 // thread -> k-block (lane & 7), row blocks wave*8 + (lane >> 3) (+32 for the second fp32 block).
+// The per-lane part of the address is a 32-bit byte offset from a wave-uniform base.
 template <typename T, bool GLU_ROWS>
 struct TransposedLoader {
   static constexpr int V = ElemTraits<T>::kVec;
   static constexpr int NB = 8 / V;  // row blocks per thread (1 for 16-bit, 2 for fp32)
-  const T *base;                    // already offset to (k = 0, row = tile row 0)
-  long long ld;
-  int kb, rb, k_valid, r_valid;
+  const char *base;                 // uniform: (k = 0, row = tile row 0)
+  long long ld_bytes;               // uniform
+  uint32_t lane_off[NB];            // (kb*V) * ld_bytes + clamped row * sizeof(T)
+  int kb, rb, k_valid;
   u32x4 regs[8];
 
-  __device__ inline void fetch(int k0) {
+  __device__ inline void setup(const T *b, long long ld, int kb_, int rb_, int k_valid_, int r_valid) {
+    base = (const char *)b;
+    ld_bytes = ld * (long long)sizeof(T);
+    kb = kb_; rb = rb_; k_valid = k_valid_;
 #pragma unroll
     for (int h = 0; h < NB; ++h) {
       int r = (rb + 32 * h) * V;
-      bool r_ok = r < r_valid;
+      if (r >= r_valid) r = 0;
+      lane_off[h] = (uint32_t)(kb * V) * (uint32_t)ld_bytes + (uint32_t)r * (uint32_t)sizeof(T);
+    }
+  }
+  template <bool TAIL>
+  __device__ inline void fetch(int k0) {
+    const char *slab = base + (long long)k0 * ld_bytes;
+#pragma unroll
+    for (int h = 0; h < NB; ++h) {
 #pragma unroll
       for (int i = 0; i < V; ++i) {
-        int k = k0 + kb * V + i;
-        u32x4 v = {0, 0, 0, 0};
-        if (r_ok && k < k_valid) v = *(const u32x4 *)(base + (long long)k * ld + r);
-        regs[h * V + i] = v;
+        if (!TAIL) {
+          regs[h * V + i] = *(const u32x4 *)(slab + i * ld_bytes + lane_off[h]);
+        } else {
+          const bool ok = k0 + kb * V + i < k_valid;
+          // a k row past the end re-reads row k0 of the slab (always valid) and is zeroed
+          const char *p = ok ? slab + i * ld_bytes + lane_off[h] : slab + (lane_off[h] - (uint32_t)(kb * V) * (uint32_t)ld_bytes);
+          u32x4 v = *(const u32x4 *)p;
+          regs[h * V + i] = ok ? v : (u32x4){0, 0, 0, 0};
+        }
       }
     }
   }
@@ -194,163 +223,112 @@ struct TransposedLoader {
   }
 };
 
-template <typename T, int A_KIND, int B_KIND, int EPI, int PROB, bool GATHER>
-__global__ __launch_bounds__(kGemmThreads) void grouped_gemm_kernel(const GemmArgs args) {
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-  constexpr int BK = kRowBytes / (int)sizeof(T);
-  constexpr bool GLU_ROWS = EPI == EPI_GLU;
-  static_assert(!(EPI == EPI_GLU) || B_KIND == OP_TRANSPOSED, "GLU epilogue expects [K,N] weights");
+// Everything a workgroup knows about its tile.
+struct TileInfo {
+  int expert, row0, rows_valid, n0, k_len, m0;
+  long long a_first;
+};
 
+// The contraction loop and the epilogue, specialised on NMI = number of 32-row blocks this wave
+// owns (0..4; partial tiles at the end of an expert's rows own fewer).
+template <typename T, int A_KIND, int B_KIND, int EPI, int PROB, int NMI, class LA, class LB>
+__device__ inline void run_tile(const GemmArgs &args, const TileInfo &ti, LA &la, LB &lb, char *lds) {
+  constexpr int BK = kRowBytes / (int)sizeof(T);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
+  constexpr int NACC = NMI > 0 ? NMI : 1;
 
-  // ---- which tile -------------------------------------------------------------------------------
-  int expert, row0, rows_valid, col_tile, k_len;
-  long long a_first = 0;  // PROB_WGRAD: first k row of the expert
-  int m0 = 0;             // PROB_WGRAD: first output row of this tile
-  {
-    int n_row_tiles = (PROB == PROB_ROWS) ? args.sched[0] : args.E * args.n_row_tiles_wgrad;
-    int total = n_row_tiles * args.n_col_tiles;
-    int total8 = (total + kXcds - 1) / kXcds * kXcds;
-    int b = blockIdx.x;
-    if (b >= total8) return;
-    int L = (b % kXcds) * (total8 / kXcds) + b / kXcds;
-    if (L >= total) return;
-    if (PROB == PROB_ROWS) {
-      const int *tiles = args.sched + kSchedHeader;
-      int t0 = L / args.n_col_tiles;
-      int gfirst = tiles[8 * t0 + 3], gcount = tiles[8 * t0 + 4];
-      int local = L - gfirst * args.n_col_tiles;
-      col_tile = local / gcount;
-      const int *te = tiles + 8 * (gfirst + local % gcount);
-      expert = te[0]; row0 = te[1]; rows_valid = te[2];
-      k_len = args.Kd;
-    } else {
-      int per_expert = args.n_row_tiles_wgrad * args.n_col_tiles;
-      expert = L / per_expert;
-      int local = L - expert * per_expert;
-      col_tile = local / args.n_row_tiles_wgrad;
-      m0 = (local % args.n_row_tiles_wgrad) * kBM;
-      row0 = 0;
-      rows_valid = min(kBM, args.Md - m0);
-      k_len = min(args.counts[expert], args.capacity);
-      a_first = args.offsets[expert];
-    }
-  }
-  const int n0 = col_tile * kBN;
-
-  // ---- loaders ------------------------------------------------------------------------------------
-  KContigLoader<T> a_k;
-  TransposedLoader<T, false> a_t;
-  KContigLoader<T> b_k;
-  TransposedLoader<T, GLU_ROWS> b_t;
-  if (A_KIND == OP_KCONTIG) {
-    a_k.base = (const T *)args.A;
-    a_k.chunk = tid & 7;
-    a_k.Kd = k_len;
+  f32x16 acc[NACC][4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      int r = min((tid >> 3) + 32 * i, rows_valid - 1);
-      long long src = row0 + r;
-      if (GATHER) src = args.a_rows[row0 + r] / args.a_div;
-      a_k.row_off[i] = src * args.lda;
-    }
-  } else {
-    a_t.base = (const T *)args.A + a_first * args.lda + m0;
-    a_t.ld = args.lda;
-    a_t.kb = lane & 7;
-    a_t.rb = wave * 8 + (lane >> 3);
-    a_t.k_valid = k_len;
-    a_t.r_valid = rows_valid;
-  }
-  if (B_KIND == OP_KCONTIG) {
-    // B element (k, n) at B[expert][n][k]: rows are output columns
-    b_k.base = (const T *)args.B + (long long)expert * args.b_expert_stride;
-    b_k.chunk = tid & 7;
-    b_k.Kd = k_len;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      int n = min(n0 + (tid >> 3) + 32 * i, args.Nd - 1);
-      b_k.row_off[i] = (long long)n * args.ldb;
-    }
-  } else {
-    if (PROB == PROB_ROWS)
-      b_t.base = (const T *)args.B + (long long)expert * args.b_expert_stride + n0;
-    else
-      b_t.base = (const T *)args.B + a_first * args.ldb + n0;
-    b_t.ld = args.ldb;
-    b_t.kb = lane & 7;
-    b_t.rb = wave * 8 + (lane >> 3);
-    b_t.k_valid = k_len;
-    b_t.r_valid = args.Nd - n0;
-  }
-
-  // LDS: stage 0 = {A, B}, stage 1 = {A, B}
-
-  f32x16 acc[4][4];
-#pragma unroll
-  for (int mi = 0; mi < 4; ++mi)
+  for (int mi = 0; mi < NACC; ++mi)
 #pragma unroll
     for (int ni = 0; ni < 4; ++ni)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
 
-  // 32-row blocks of the tile are dealt alternately to the two wave rows; blocks past the valid
-  // rows are skipped.
-  const int n_blocks32 = (rows_valid + 31) >> 5;
-  const int n_mi = (n_blocks32 - wm + 1) >> 1;
-  const int n_slabs = (k_len + BK - 1) / BK;
+  const int n_slabs = (ti.k_len + BK - 1) / BK;
 
-  auto fetch = [&](int s) {
-    if (A_KIND == OP_KCONTIG) a_k.fetch(s * BK); else a_t.fetch(s * BK);
-    if (B_KIND == OP_KCONTIG) b_k.fetch(s * BK); else b_t.fetch(s * BK);
-  };
   auto commit = [&](int buf) {
     char *tA = lds + buf * (2 * kTileBytes), *tB = tA + kTileBytes;
-    if (A_KIND == OP_KCONTIG) a_k.commit(tA, tid); else a_t.commit(tA);
-    if (B_KIND == OP_KCONTIG) b_k.commit(tB, tid); else b_t.commit(tB);
+    if constexpr (A_KIND == OP_KCONTIG) la.commit(tA, tid); else la.commit(tA);
+    if constexpr (B_KIND == OP_KCONTIG) lb.commit(tB, tid); else lb.commit(tB);
+  };
+  // MFMA operands of k-step ks+1 are read from LDS while the MFMAs of k-step ks run; the scheduling
+  // barriers keep the compiler from sinking the reads next to their first use.
+  auto load_frags = [&](const char *tA, const char *tB, int ks, u32x4 (&af)[NACC], u32x4 (&bf)[4]) {
+    const int chunk = ks * 2 + (lane >> 5);
+#pragma unroll
+    for (int ni = 0; ni < 4; ++ni) {
+      int row = wn * 128 + ni * 32 + (lane & 31);
+      bf[ni] = *(const u32x4 *)(tB + lds_chunk_off(row, chunk));
+    }
+#pragma unroll
+    for (int mi = 0; mi < NMI; ++mi) {
+      int row = (mi * 2 + wm) * 32 + (lane & 31);
+      af[mi] = *(const u32x4 *)(tA + lds_chunk_off(row, chunk));
+    }
+  };
+  auto mma = [&](const u32x4 (&af)[NACC], const u32x4 (&bf)[4]) {
+#pragma unroll
+    for (int mi = 0; mi < NMI; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < 4; ++ni) Mma<T>::run(af[mi], bf[ni], acc[mi][ni]);
+  };
+  auto compute = [&](int buf) {
+    const char *tA = lds + buf * (2 * kTileBytes), *tB = tA + kTileBytes;
+    u32x4 af0[NACC], bf0[4], af1[NACC], bf1[4];
+    load_frags(tA, tB, 0, af0, bf0);
+    __builtin_amdgcn_sched_barrier(0);
+    load_frags(tA, tB, 1, af1, bf1);
+    mma(af0, bf0);
+    __builtin_amdgcn_sched_barrier(0);
+    load_frags(tA, tB, 2, af0, bf0);
+    mma(af1, bf1);
+    __builtin_amdgcn_sched_barrier(0);
+    load_frags(tA, tB, 3, af1, bf1);
+    mma(af0, bf0);
+    __builtin_amdgcn_sched_barrier(0);
+    mma(af1, bf1);
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   if (n_slabs > 0) {
-    fetch(0);
+    if (n_slabs == 1) { la.template fetch<true>(0); lb.template fetch<true>(0); }
+    else { la.template fetch<false>(0); lb.template fetch<false>(0); }
     commit(0);
   }
   __syncthreads();
-
-  for (int s = 0; s < n_slabs; ++s) {
-    const int buf = s & 1;
-    if (s + 1 < n_slabs) fetch(s + 1);
-    const char *tA = lds + buf * (2 * kTileBytes), *tB = tA + kTileBytes;
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const int chunk = ks * 2 + (lane >> 5);
-      u32x4 bf[4];
-#pragma unroll
-      for (int ni = 0; ni < 4; ++ni) {
-        int row = wn * 128 + ni * 32 + (lane & 31);
-        bf[ni] = *(const u32x4 *)(tB + lds_chunk_off(row, chunk));
-      }
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi) {
-        if (mi < n_mi) {
-          int row = (mi * 2 + wm) * 32 + (lane & 31);
-          u32x4 af = *(const u32x4 *)(tA + lds_chunk_off(row, chunk));
-#pragma unroll
-          for (int ni = 0; ni < 4; ++ni) Mma<T>::run(af, bf[ni], acc[mi][ni]);
-        }
-      }
-    }
-    if (s + 1 < n_slabs) commit(buf ^ 1);
+  int s = 0;
+  for (; s + 2 < n_slabs; ++s) {  // slab s+1 is a full one
+    la.template fetch<false>((s + 1) * BK);
+    lb.template fetch<false>((s + 1) * BK);
+    __builtin_amdgcn_sched_barrier(0);  // the loads of the next slab are issued before this slab's MFMAs
+    compute(s & 1);
+    commit((s & 1) ^ 1);
     __syncthreads();
   }
+  if (s + 1 < n_slabs) {  // slab s+1 is the last one and may be partial
+    la.template fetch<true>((s + 1) * BK);
+    lb.template fetch<true>((s + 1) * BK);
+    __builtin_amdgcn_sched_barrier(0);
+    compute(s & 1);
+    commit((s & 1) ^ 1);
+    __syncthreads();
+    ++s;
+  }
+  if (s < n_slabs) compute(s & 1);
+
+  if constexpr (NMI == 0) return;
 
   // ---- epilogue -------------------------------------------------------------------------------------
   // acc[mi][ni][v]: tile row (mi*2+wm)*32 + 8*(v/4) + 4*(lane/32) + v%4, LDS column row wn*128 + ni*32 + lane%32
   const int lcol = lane & 31;
   const int rsub = (lane >> 5) * 4;
-  if (EPI == EPI_STORE) {
-    T *C = (T *)args.C;
-    long long c_base = (PROB == PROB_WGRAD) ? (long long)expert * args.c_expert_stride : 0;
+  const int expert = ti.expert, rows_valid = ti.rows_valid, n0 = ti.n0;
+  const long long out_row0 = (PROB == PROB_WGRAD) ? ti.m0 : ti.row0;
+  const bool full = rows_valid == kBM && n0 + kBN <= args.Nd;
+  if constexpr (EPI == EPI_STORE) {
+    T *C = (T *)args.C + ((PROB == PROB_WGRAD) ? (long long)expert * args.c_expert_stride : 0);
 #pragma unroll
     for (int ni = 0; ni < 4; ++ni) {
       int col = n0 + wn * 128 + ni * 32 + lcol;
@@ -359,15 +337,18 @@ __global__ __launch_bounds__(kGemmThreads) void grouped_gemm_kernel(const GemmAr
       if (args.bias != nullptr && col_ok)
         bias = ElemTraits<T>::to_f32(((const T *)args.bias)[(long long)expert * args.Nd + col]);
 #pragma unroll
-      for (int mi = 0; mi < 4; ++mi) {
-        if (mi < n_mi) {
+      for (int mi = 0; mi < NMI; ++mi) {
+        T *Cp = C + (out_row0 + (mi * 2 + wm) * 32 + rsub) * args.ldc + col;
+        if (full) {
+#pragma unroll
+          for (int v = 0; v < 16; ++v)
+            Cp[(long long)(8 * (v >> 2) + (v & 3)) * args.ldc] = ElemTraits<T>::from_f32(acc[mi][ni][v] + bias);
+        } else {
 #pragma unroll
           for (int v = 0; v < 16; ++v) {
             int r = (mi * 2 + wm) * 32 + 8 * (v >> 2) + rsub + (v & 3);
-            if (col_ok && r < rows_valid) {
-              long long orow = (PROB == PROB_WGRAD) ? (m0 + r) : (row0 + r);
-              C[c_base + orow * args.ldc + col] = ElemTraits<T>::from_f32(acc[mi][ni][v] + bias);
-            }
+            if (col_ok && r < rows_valid)
+              Cp[(long long)(8 * (v >> 2) + (v & 3)) * args.ldc] = ElemTraits<T>::from_f32(acc[mi][ni][v] + bias);
           }
         }
       }
@@ -381,32 +362,127 @@ __global__ __launch_bounds__(kGemmThreads) void grouped_gemm_kernel(const GemmAr
       int pair = (n0 + wn * 128) / 2 + np * 32 + lcol;  // index of the (gate, up) pair = act column
       bool col_ok = 2 * pair + 1 < args.Nd;
       float bg = 0.0f, bu = 0.0f;
-      if (EPI == EPI_GLU && args.bias != nullptr && col_ok) {
+      if (args.bias != nullptr && col_ok) {
         const T *bp = (const T *)args.bias + (long long)expert * args.Nd + 2 * pair;
         bg = ElemTraits<T>::to_f32(bp[0]);
         bu = ElemTraits<T>::to_f32(bp[1]);
       }
 #pragma unroll
-      for (int mi = 0; mi < 4; ++mi) {
-        if (mi < n_mi) {
+      for (int mi = 0; mi < NMI; ++mi) {
 #pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            int r = (mi * 2 + wm) * 32 + 8 * (v >> 2) + rsub + (v & 3);
-            if (col_ok && r < rows_valid) {
-              long long orow = row0 + r;
-              if (EPI == EPI_GLU) {
-                float G = acc[mi][np][v] + bg, U = acc[mi][np + 2][v] + bu;
-                C[orow * args.ldc + pair] = ElemTraits<T>::from_f32(glu_forward(G, U));
-                if (P != nullptr) {
-                  P[orow * args.Nd + 2 * pair] = ElemTraits<T>::from_f32(G);
-                  P[orow * args.Nd + 2 * pair + 1] = ElemTraits<T>::from_f32(U);
-                }
-              }
+        for (int v = 0; v < 16; ++v) {
+          int r = (mi * 2 + wm) * 32 + 8 * (v >> 2) + rsub + (v & 3);
+          if (full || (col_ok && r < rows_valid)) {
+            long long orow = out_row0 + r;
+            float G = acc[mi][np][v] + bg, U = acc[mi][np + 2][v] + bu;
+            C[orow * args.ldc + pair] = ElemTraits<T>::from_f32(glu_forward(G, U));
+            if (P != nullptr) {
+              P[orow * args.Nd + 2 * pair] = ElemTraits<T>::from_f32(G);
+              P[orow * args.Nd + 2 * pair + 1] = ElemTraits<T>::from_f32(U);
             }
           }
         }
       }
     }
+  }
+}
+
+template <typename T, int A_KIND, int B_KIND, int EPI, int PROB, bool GATHER>
+__global__ __launch_bounds__(kGemmThreads) void grouped_gemm_kernel(const GemmArgs args) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  constexpr int V = ElemTraits<T>::kVec;
+  constexpr bool GLU_ROWS = EPI == EPI_GLU;
+  static_assert(!(EPI == EPI_GLU) || B_KIND == OP_TRANSPOSED, "GLU epilogue expects [K,N] weights");
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1;
+
+  // ---- which tile -------------------------------------------------------------------------------
+  TileInfo ti;
+  ti.a_first = 0;
+  ti.m0 = 0;
+  {
+    int n_row_tiles = (PROB == PROB_ROWS) ? args.sched[0] : args.E * args.n_row_tiles_wgrad;
+    int total = n_row_tiles * args.n_col_tiles;
+    int total8 = (total + kXcds - 1) / kXcds * kXcds;
+    int b = blockIdx.x;
+    if (b >= total8) return;
+    int L = (b % kXcds) * (total8 / kXcds) + b / kXcds;
+    if (L >= total) return;
+    int col_tile;
+    if (PROB == PROB_ROWS) {
+      const int *tiles = args.sched + kSchedHeader;
+      int t0 = L / args.n_col_tiles;
+      int gfirst = tiles[8 * t0 + 3], gcount = tiles[8 * t0 + 4];
+      int local = L - gfirst * args.n_col_tiles;
+      col_tile = local / gcount;
+      const int *te = tiles + 8 * (gfirst + local % gcount);
+      ti.expert = te[0]; ti.row0 = te[1]; ti.rows_valid = te[2];
+      ti.k_len = args.Kd;
+    } else {
+      int per_expert = args.n_row_tiles_wgrad * args.n_col_tiles;
+      ti.expert = L / per_expert;
+      int local = L - ti.expert * per_expert;
+      col_tile = local / args.n_row_tiles_wgrad;
+      ti.m0 = (local % args.n_row_tiles_wgrad) * kBM;
+      ti.row0 = 0;
+      ti.rows_valid = min(kBM, args.Md - ti.m0);
+      ti.k_len = min(args.counts[ti.expert], args.capacity);
+      ti.a_first = args.offsets[ti.expert];
+    }
+    ti.n0 = col_tile * kBN;
+  }
+
+  // ---- loaders ------------------------------------------------------------------------------------
+  typedef typename std::conditional<A_KIND == OP_KCONTIG, KContigLoader<T>, TransposedLoader<T, false>>::type LA;
+  typedef typename std::conditional<B_KIND == OP_KCONTIG, KContigLoader<T>, TransposedLoader<T, GLU_ROWS>>::type LB;
+  LA la;
+  LB lb;
+  if constexpr (A_KIND == OP_KCONTIG) {
+    la.chunk = tid & 7;
+    la.Kd = ti.k_len;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int r = min((tid >> 3) + 32 * i, ti.rows_valid - 1);
+      // byte offsets fit 32 bits: rows of a tile are near its first row, and gathered sources are
+      // checked on the host to span less than 4 GB
+      long long src = r;
+      if (GATHER) src = args.a_rows[ti.row0 + r] / args.a_div;
+      la.row_off[i] = (uint32_t)((src * args.lda + (tid & 7) * V) * (long long)sizeof(T));
+    }
+    la.base = (const char *)((const T *)args.A + (GATHER ? 0ll : (long long)ti.row0 * args.lda));
+  } else {
+    la.setup((const T *)args.A + ti.a_first * args.lda + ti.m0, args.lda, lane & 7, wave * 8 + (lane >> 3), ti.k_len,
+             ti.rows_valid);
+  }
+  if constexpr (B_KIND == OP_KCONTIG) {
+    // B element (k, n) at B[expert][n][k]: rows are output columns
+    const T *bb = (const T *)args.B + (long long)ti.expert * args.b_expert_stride;
+    lb.chunk = tid & 7;
+    lb.Kd = ti.k_len;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int n = min(ti.n0 + (tid >> 3) + 32 * i, args.Nd - 1);
+      lb.row_off[i] = (uint32_t)(((long long)n * args.ldb + (tid & 7) * V) * (long long)sizeof(T));
+    }
+    lb.base = (const char *)bb;
+  } else {
+    const T *bb = (PROB == PROB_ROWS) ? (const T *)args.B + (long long)ti.expert * args.b_expert_stride + ti.n0
+                                      : (const T *)args.B + ti.a_first * args.ldb + ti.n0;
+    lb.setup(bb, args.ldb, lane & 7, wave * 8 + (lane >> 3), ti.k_len, args.Nd - ti.n0);
+  }
+
+  // 32-row blocks of the tile are dealt alternately to the two wave rows; blocks past the valid
+  // rows are skipped.  The branch is uniform per wave, and every wave of the workgroup runs the
+  // same number of slabs and barriers whatever its block count.
+  const int n_blocks32 = (ti.rows_valid + 31) >> 5;
+  const int n_mi = (n_blocks32 - wm + 1) >> 1;
+  switch (n_mi) {
+    case 4: run_tile<T, A_KIND, B_KIND, EPI, PROB, 4>(args, ti, la, lb, lds); break;
+    case 3: run_tile<T, A_KIND, B_KIND, EPI, PROB, 3>(args, ti, la, lb, lds); break;
+    case 2: run_tile<T, A_KIND, B_KIND, EPI, PROB, 2>(args, ti, la, lb, lds); break;
+    case 1: run_tile<T, A_KIND, B_KIND, EPI, PROB, 1>(args, ti, la, lb, lds); break;
+    default: run_tile<T, A_KIND, B_KIND, EPI, PROB, 0>(args, ti, la, lb, lds); break;
   }
 }
 
