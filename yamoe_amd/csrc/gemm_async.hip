@@ -1,0 +1,394 @@
+// Grouped expert GEMMs for 16-bit data on gfx950, asynchronous-copy pipeline.
+//
+// Same tiling as gemm.hip (256x256 output tile, 4 wavefronts 2x2, 32x32x16 MFMA, fp32 accumulate)
+// but operands never pass through vector registers on their way to LDS:
+//
+//  * Global -> LDS copies are `global_load_lds_dwordx4`: every lane names its own 16-byte source and
+//    the 64 lanes of a wave fill 1 KB of LDS in lane order.  The contraction is cut into slabs of
+//    32; four slab buffers (4 x 32 KB) rotate, and a slab is requested four slabs (about 3000 MFMA
+//    cycles) before it is consumed, which covers HBM latency with one wave per SIMD.
+//  * An operand whose rows are k-contiguous in memory ([row][k]) keeps that layout in LDS
+//    (64 bytes per row) and is read with one 16-byte ds_read per MFMA operand.
+//  * The forward weights are [k][n] in memory and stay [k][n] in LDS (512 bytes per k row);
+//    MFMA operands are read with `ds_read_b64_tr_b16`, the LDS transpose read of gfx950, which
+//    hands lane i of a 16-lane group column n0+i for 4 consecutive k.  No register transpose, no
+//    LDS store instruction, no staging registers.
+//  * LDS swizzles are applied on the global side (a lane picks which 16-byte piece it fetches), as
+//    the LDS side of an asynchronous copy is fixed to lane order:
+//        [row][k] tiles: piece c of row r sits at position c ^ ((r >> 2) & 3)
+//        [k][n]  tiles: piece c of row k sits at position c ^ ((k & 3) << 2)
+//    so that both kinds of MFMA operand reads touch every bank once.
+//  * Software pipeline per slab (two k-steps of 16): the operands of the second k-step are read
+//    while the MFMAs of the first run; then the wave waits for the next slab's copies, one
+//    workgroup barrier, the freed buffer is re-filled with slab s+4, the first operands of slab
+//    s+1 are read, and the MFMAs of the second k-step run.  All LDS and HBM latency sits behind
+//    MFMAs; only the barrier itself is exposed.
+//
+// The interleaved (gate, up) columns of the clamped SwiGLU (csrc/moe.cpp:164-180) end up in
+// neighbouring lanes of one accumulator tile; the epilogue swaps them with one DPP move per pair.
+//
+// Requirements: contraction length a multiple of 32, leading dimensions multiples of 8 elements.
+// Other shapes and fp32 use gemm.hip.
+#include <type_traits>
+
+#include "common.h"
+
+namespace yamoe {
+
+namespace async {
+
+constexpr int kBM = 256, kBN = 256, kBK = 32;
+constexpr int kThreads = 256;
+constexpr int kStages = 4;
+constexpr int kOperandBytes = 16384;           // one operand, one slab
+constexpr int kStageBytes = 2 * kOperandBytes;  // A then B
+constexpr int kLds = kStages * kStageBytes;     // 128 KB
+constexpr int kXcds = 8;
+
+static_assert(kBM == kRowTile, "row tiles of the schedule must match the GEMM tile");
+
+enum { EPI_STORE = 0, EPI_GLU = 1 };
+
+struct Args {
+  const void *A;        // [rows, lda], k-contiguous
+  const void *B;        // [E, Kd, Nd] ([k][n] per expert)
+  const void *bias;     // [E, Nd] or null
+  void *C;              // EPI_STORE: [rows, ldc]; EPI_GLU: act [rows, Nd/2]
+  void *C2;             // EPI_GLU: optional pre-activations [rows, Nd]
+  const int *a_rows;    // optional gather of A rows: source row = a_rows[p] / a_div
+  const int *sched;
+  int a_div, Kd, Nd, lda, ldb, ldc, n_col_tiles;
+  long long b_expert_stride;
+};
+
+template <typename T> struct Mma;
+template <> struct Mma<bf16_t> {
+  __device__ static inline void run(const u32x4 &a, const u32x4 &b, f32x16 &c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma<f16_t> {
+  __device__ static inline void run(const u32x4 &a, const u32x4 &b, f32x16 &c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+
+// 16 bytes per lane from global memory straight into LDS at lds_base + lane * 16.
+__device__ inline void copy16_to_lds(const void *uniform_base, uint32_t lane_byte_off, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(lane_byte_off), "s"(uniform_base), "s"(lds_base)
+               : "memory");
+}
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+
+// LDS transpose read: lane i of each 16-lane group receives, for j = 0..3, the 16-bit element
+// (i % 4) of the 8 bytes addressed by lane 4*j + i/4 of the group.
+__device__ inline u32x2 lds_read_tr16(const char *p) {
+  s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)p);
+  return __builtin_bit_cast(u32x2, v);
+}
+
+// Wait until at most `newer` slabs' worth of this wave's copies (8 each) are still in flight.
+__device__ inline void wait_copies(int newer) {
+  switch (newer) {
+    case 4: asm volatile("s_waitcnt vmcnt(32)" ::: "memory"); break;
+    case 3: asm volatile("s_waitcnt vmcnt(24)" ::: "memory"); break;
+    case 2: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
+    case 1: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+    default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+  }
+}
+
+struct TileInfo {
+  int expert, row0, rows_valid, n0;
+};
+
+template <typename T, int EPI, int NMI>
+__device__ inline void run_tile(const Args &args, const TileInfo &ti, const char *a_base, const uint32_t (&a_off)[4],
+                                const char *b_base, const uint32_t (&b_off)[4], long long b_ld_bytes) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  constexpr int NACC = NMI > 0 ? NMI : 1;
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)lds;  // LDS byte address of the first slab buffer
+
+  f32x16 acc[NACC][4];
+#pragma unroll
+  for (int mi = 0; mi < NACC; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < 4; ++ni)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
+
+  const int n_slabs = args.Kd / kBK;
+
+  // ---- copy issue ----------------------------------------------------------------------------------
+  // A: this wave fills rows 64*wave + 16*i + (lane >> 2); B: k rows 8*wave + 2*i + (lane >> 5).
+  auto issue = [&](int slab) {
+    const uint32_t stage = lds0 + (uint32_t)(slab % kStages) * kStageBytes;
+    const char *ab = a_base + (long long)slab * (kBK * (int)sizeof(T));
+    const char *bb = b_base + (long long)slab * kBK * b_ld_bytes;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      copy16_to_lds(ab, a_off[i], __builtin_amdgcn_readfirstlane(stage + (uint32_t)(64 * wave + 16 * i) * 64u));
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      copy16_to_lds(bb, b_off[i],
+                    __builtin_amdgcn_readfirstlane(stage + kOperandBytes + (uint32_t)(8 * wave + 2 * i) * 512u));
+  };
+
+  // ---- MFMA operand reads ----------------------------------------------------------------------------
+  // A operand (block mi, k-step ks): row (mi*2+wm)*32 + lane%32, piece ks*2 + lane/32.
+  const int rl = lane & 31, g = lane >> 5;
+  int a_rd[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks)
+    a_rd[ks] = (wm * 32 + rl) * 64 + (((ks * 2 + g) ^ ((rl >> 2) & 3)) << 4);
+  // B operand (column block ni, k-step ks, half h): k = ks*16 + g*8 + h*4 + j, 4 columns at
+  // wn*128 + ni*32 + 16*((lane>>4)&1) + 4*q, where j = (lane&15)>>2 and q = lane&3.
+  const int j4 = (lane & 15) >> 2, q4 = lane & 3;
+  int b_rd[4];
+#pragma unroll
+  for (int ni = 0; ni < 4; ++ni) {
+    int col = wn * 128 + ni * 32 + 16 * ((lane >> 4) & 1) + 4 * q4;
+    int piece = (col >> 3) ^ (j4 << 2);
+    b_rd[ni] = kOperandBytes + (g * 8 + j4) * 512 + (piece << 4) + (col & 7) * 2;
+  }
+
+  u32x4 fa0[NACC], fa1[NACC], fb0[4], fb1[4];
+  auto read_frags = [&](const char *stage, int ks, u32x4 (&fa)[NACC], u32x4 (&fb)[4]) {
+#pragma unroll
+    for (int ni = 0; ni < 4; ++ni) {
+      u32x2 lo = lds_read_tr16(stage + b_rd[ni] + ks * 8192);
+      u32x2 hi = lds_read_tr16(stage + b_rd[ni] + ks * 8192 + 2048);
+      fb[ni] = (u32x4){lo[0], lo[1], hi[0], hi[1]};
+    }
+#pragma unroll
+    for (int mi = 0; mi < NMI; ++mi) fa[mi] = *(const u32x4 *)(stage + a_rd[ks] + mi * 4096);
+  };
+  auto mma = [&](const u32x4 (&fa)[NACC], const u32x4 (&fb)[4]) {
+#pragma unroll
+    for (int mi = 0; mi < NMI; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < 4; ++ni) Mma<T>::run(fa[mi], fb[ni], acc[mi][ni]);
+  };
+
+  // ---- pipeline -----------------------------------------------------------------------------------------
+  const int n_pro = n_slabs < kStages ? n_slabs : kStages;
+  for (int d = 0; d < n_pro; ++d) issue(d);
+  wait_copies(n_pro - 1);
+  __syncthreads();
+  read_frags(lds, 0, fa0, fb0);
+
+  for (int s = 0; s < n_slabs; ++s) {
+    const char *stage = lds + (s % kStages) * kStageBytes;
+    const char *next_stage = lds + ((s + 1) % kStages) * kStageBytes;
+    read_frags(stage, 1, fa1, fb1);
+    mma(fa0, fb0);
+    __builtin_amdgcn_sched_barrier(0);
+    if (s + 1 < n_slabs) {
+      int last = n_slabs - 1 < s + kStages - 1 ? n_slabs - 1 : s + kStages - 1;
+      wait_copies(last - (s + 1));  // slab s+1 has landed (this wave's share)
+    }
+    // The barrier waits for this wave's LDS reads first, so after it nobody reads slab s's buffer any
+    // more and everybody's share of slab s+1 is visible.
+    __syncthreads();
+    if (s + kStages < n_slabs) issue(s + kStages);
+    if (s + 1 < n_slabs) read_frags(next_stage, 0, fa0, fb0);
+    mma(fa1, fb1);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  if constexpr (NMI == 0) return;
+
+  // ---- epilogue -------------------------------------------------------------------------------------
+  // acc[mi][ni][v]: tile row (mi*2+wm)*32 + 8*(v/4) + 4*(lane/32) + v%4, tile column wn*128 + ni*32 + lane%32
+  const int rsub = g * 4;
+  const int expert = ti.expert, rows_valid = ti.rows_valid, n0 = ti.n0;
+  const long long out_row0 = ti.row0;
+  const bool full = rows_valid == kBM && n0 + kBN <= args.Nd;
+  if constexpr (EPI == EPI_STORE) {
+    T *C = (T *)args.C;
+#pragma unroll
+    for (int ni = 0; ni < 4; ++ni) {
+      int col = n0 + wn * 128 + ni * 32 + rl;
+      bool col_ok = col < args.Nd;
+      float bias = 0.0f;
+      if (args.bias != nullptr && col_ok)
+        bias = ElemTraits<T>::to_f32(((const T *)args.bias)[(long long)expert * args.Nd + col]);
+#pragma unroll
+      for (int mi = 0; mi < NMI; ++mi) {
+        T *Cp = C + (out_row0 + (mi * 2 + wm) * 32 + rsub) * args.ldc + col;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          int r = (mi * 2 + wm) * 32 + 8 * (v >> 2) + rsub + (v & 3);
+          if (full || (col_ok && r < rows_valid))
+            Cp[(long long)(8 * (v >> 2) + (v & 3)) * args.ldc] = ElemTraits<T>::from_f32(acc[mi][ni][v] + bias);
+        }
+      }
+    }
+  } else {
+    // Even lanes hold gate columns, odd lanes the matching up columns.  For each pair of accumulator
+    // rows (v, v+1) the even lane finishes row v and the odd lane row v+1 after one DPP swap.
+    T *C = (T *)args.C;
+    T *P = (T *)args.C2;
+    const bool odd = lane & 1;
+#pragma unroll
+    for (int ni = 0; ni < 4; ++ni) {
+      int col = n0 + wn * 128 + ni * 32 + (rl & ~1);  // the gate column of this lane's pair
+      int pair = col >> 1;
+      bool col_ok = col + 1 < args.Nd;
+      float bg = 0.0f, bu = 0.0f;
+      if (args.bias != nullptr && col_ok) {
+        const T *bp = (const T *)args.bias + (long long)expert * args.Nd + col;
+        bg = ElemTraits<T>::to_f32(bp[0]);
+        bu = ElemTraits<T>::to_f32(bp[1]);
+      }
+#pragma unroll
+      for (int mi = 0; mi < NMI; ++mi) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          float xe = acc[mi][ni][2 * u], xo = acc[mi][ni][2 * u + 1];
+          float send = odd ? xe : xo;
+          float recv = __builtin_bit_cast(
+              float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, send), 0xB1 /* quad_perm [1,0,3,2] */, 0xF, 0xF, true));
+          float G = (odd ? recv : xe) + bg, U = (odd ? xo : recv) + bu;
+          int v = 2 * u + (odd ? 1 : 0);
+          int r = (mi * 2 + wm) * 32 + 8 * (v >> 2) + rsub + (v & 3);
+          if (full || (col_ok && r < rows_valid)) {
+            long long orow = out_row0 + r;
+            C[orow * args.ldc + pair] = ElemTraits<T>::from_f32(glu_forward(G, U));
+            if (P != nullptr) {
+              P[orow * args.Nd + col] = ElemTraits<T>::from_f32(G);
+              P[orow * args.Nd + col + 1] = ElemTraits<T>::from_f32(U);
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+template <typename T, int EPI, bool GATHER>
+__global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1;
+
+  TileInfo ti;
+  {
+    int n_row_tiles = args.sched[0];
+    int total = n_row_tiles * args.n_col_tiles;
+    int total8 = (total + kXcds - 1) / kXcds * kXcds;
+    int b = blockIdx.x;
+    if (b >= total8) return;
+    int L = (b % kXcds) * (total8 / kXcds) + b / kXcds;
+    if (L >= total) return;
+    const int *tiles = args.sched + kSchedHeader;
+    int t0 = L / args.n_col_tiles;
+    int gfirst = tiles[8 * t0 + 3], gcount = tiles[8 * t0 + 4];
+    int local = L - gfirst * args.n_col_tiles;
+    int col_tile = local / gcount;
+    const int *te = tiles + 8 * (gfirst + local % gcount);
+    ti.expert = te[0]; ti.row0 = te[1]; ti.rows_valid = te[2];
+    ti.n0 = col_tile * kBN;
+  }
+
+  // A copies: rows 64*wave + 16*i + (lane >> 2); LDS position lane & 3 holds piece pos ^ ((row >> 2) & 3)
+  uint32_t a_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int row = 64 * wave + 16 * i + (lane >> 2);
+    int piece = (lane & 3) ^ ((row >> 2) & 3);
+    int r = min(row, ti.rows_valid - 1);
+    long long src = r;
+    if (GATHER) src = args.a_rows[ti.row0 + r] / args.a_div;
+    a_off[i] = (uint32_t)((src * args.lda + piece * 8) * (long long)sizeof(T));
+  }
+  const char *a_base = (const char *)((const T *)args.A + (GATHER ? 0ll : (long long)ti.row0 * args.lda));
+
+  // B copies: k rows 8*wave + 2*i + (lane >> 5); LDS position lane & 31 holds piece pos ^ ((k & 3) << 2)
+  const long long b_ld_bytes = (long long)args.ldb * (long long)sizeof(T);
+  uint32_t b_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int k = 8 * wave + 2 * i + (lane >> 5);
+    int piece = (lane & 31) ^ ((k & 3) << 2);
+    int col = ti.n0 + piece * 8;
+    if (col >= args.Nd) col = ti.n0;  // columns past the end re-read valid ones; never stored
+    b_off[i] = (uint32_t)(k * b_ld_bytes + (long long)(col - ti.n0) * (long long)sizeof(T));
+  }
+  const char *b_base = (const char *)((const T *)args.B + (long long)ti.expert * args.b_expert_stride + ti.n0);
+
+  const int n_blocks32 = (ti.rows_valid + 31) >> 5;
+  const int n_mi = (n_blocks32 - wm + 1) >> 1;
+  switch (n_mi) {
+    case 4: run_tile<T, EPI, 4>(args, ti, a_base, a_off, b_base, b_off, b_ld_bytes); break;
+    case 3: run_tile<T, EPI, 3>(args, ti, a_base, a_off, b_base, b_off, b_ld_bytes); break;
+    case 2: run_tile<T, EPI, 2>(args, ti, a_base, a_off, b_base, b_off, b_ld_bytes); break;
+    case 1: run_tile<T, EPI, 1>(args, ti, a_base, a_off, b_base, b_off, b_ld_bytes); break;
+    default: run_tile<T, EPI, 0>(args, ti, a_base, a_off, b_base, b_off, b_ld_bytes); break;
+  }
+}
+
+template <typename T, int EPI, bool GATHER>
+static int launch(const Args &args, int max_row_tiles, hipStream_t stream) {
+  auto kernel = gemm_async_kernel<T, EPI, GATHER>;
+  static bool attr_done = false;  // benign race: the attribute call is idempotent
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(MaxDynamicSharedMemorySize=%d): %s", kLds, hipGetErrorString(e));
+      return (int)e;
+    }
+    attr_done = true;
+  }
+  long long total = (long long)max_row_tiles * args.n_col_tiles;
+  if (total <= 0) return 0;
+  total = (total + kXcds - 1) / kXcds * kXcds;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(kThreads), kLds, stream, args);
+  return check_launch("gemm_async_kernel");
+}
+
+}  // namespace async
+
+// True when the asynchronous-copy kernels can take this product.
+bool gemm_async_supported(int Kd, int Nd, int lda, int ldb, long long a_span_bytes) {
+  return Kd % async::kBK == 0 && Kd >= async::kBK && Nd % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 &&
+         a_span_bytes < (1ll << 32);
+}
+
+template <typename T>
+int gemm_async_gate_up(const void *x, const int *sorted_idx, const void *w, const void *bias, void *act, void *pre,
+                       const void *sched, int N, int K, int E, int H, int I, hipStream_t stream) {
+  async::Args a = {};
+  a.A = x; a.B = w; a.bias = bias; a.C = act; a.C2 = pre;
+  a.a_rows = sorted_idx; a.a_div = K; a.sched = (const int *)sched;
+  a.Kd = H; a.Nd = 2 * I; a.lda = H; a.ldb = 2 * I; a.ldc = I;
+  a.b_expert_stride = (long long)H * 2 * I;
+  a.n_col_tiles = ceil_div(2 * I, async::kBN);
+  return async::launch<T, async::EPI_GLU, true>(a, sched_max_row_tiles(N, E), stream);
+}
+
+template <typename T>
+int gemm_async_down(const void *act, const void *w, const void *bias, void *y, const void *sched, int N, int E, int H,
+                    int I, hipStream_t stream) {
+  async::Args a = {};
+  a.A = act; a.B = w; a.bias = bias; a.C = y; a.sched = (const int *)sched;
+  a.Kd = I; a.Nd = H; a.lda = I; a.ldb = H; a.ldc = H;
+  a.b_expert_stride = (long long)I * H;
+  a.n_col_tiles = ceil_div(H, async::kBN);
+  return async::launch<T, async::EPI_STORE, false>(a, sched_max_row_tiles(N, E), stream);
+}
+
+#define YAMOE_INSTANTIATE_ASYNC(T)                                                                               \
+  template int gemm_async_gate_up<T>(const void *, const int *, const void *, const void *, void *, void *,      \
+                                     const void *, int, int, int, int, int, hipStream_t);                        \
+  template int gemm_async_down<T>(const void *, const void *, const void *, void *, const void *, int, int, int, \
+                                  int, hipStream_t);
+YAMOE_INSTANTIATE_ASYNC(bf16_t)
+YAMOE_INSTANTIATE_ASYNC(f16_t)
+
+}  // namespace yamoe
