@@ -99,3 +99,39 @@ def test_permute_and_combine(gpu, dtype, T, K, E, H):
     all_dropped = (invp < 0).all(axis=1)
     if all_dropped.any():
         assert torch.all(got[torch.from_numpy(all_dropped)] == 0)
+
+
+@pytest.mark.parametrize("N,E,C,stream_rows", [(256, 128, 64, 16), (16384, 32, 4096, 16), (65536, 128, 300, 16),
+                                               (1000, 700, 5, 0), (40, 3, 40, 16)])
+def test_schedule_lists(gpu, N, E, C, stream_rows):
+    """The device-built work lists: experts with 1..stream_rows kept rows in the streaming list, the
+    rest cut into 256-row tiles, both in expert order, none dropped, none duplicated."""
+    from yamoe_amd import _cabi
+    rng = np.random.default_rng(N * 7 + E)
+    p = rng.random(E) ** 4
+    ids = rng.choice(E, size=N, p=p / p.sum())
+    r = O.route(ids, E, C)
+    counts = torch.from_numpy(r["counts"]).to(gpu)
+    offsets = torch.from_numpy(r["offsets"]).to(gpu)
+    sched = _cabi.build_schedule(counts, offsets, N, C, stream_rows).cpu().numpy()
+    want_tiles, want_small = [], []
+    for e in range(E):
+        kept = min(int(r["counts"][e]), C)
+        if kept == 0:
+            continue
+        first = int(r["offsets"][e])
+        if kept <= stream_rows:
+            want_small.append((e, first, kept))
+        else:
+            g0, n = len(want_tiles), -(-kept // 256)
+            for t in range(n):
+                want_tiles.append((e, first + 256 * t, min(256, kept - 256 * t), g0, n))
+    n_tiles, n_small, n_active, n_kept = sched[:4]
+    assert n_tiles == len(want_tiles) and n_small == len(want_small)
+    assert n_active == int((np.minimum(r["counts"], C) > 0).sum())
+    assert n_kept == int(np.minimum(r["counts"], C).sum())
+    max_tiles = N // 256 + min(N, E) + 1
+    tiles = sched[8:8 + 8 * n_tiles].reshape(-1, 8)[:, :5]
+    assert [tuple(t) for t in tiles.tolist()] == want_tiles
+    small = sched[8 + 8 * max_tiles:8 + 8 * max_tiles + 4 * n_small].reshape(-1, 4)[:, :3]
+    assert [tuple(t) for t in small.tolist()] == want_small

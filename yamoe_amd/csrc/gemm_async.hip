@@ -39,10 +39,12 @@ namespace async {
 
 constexpr int kBM = 256, kBN = 256, kBK = 32;
 constexpr int kThreads = 256;
-constexpr int kStages = 4;
-constexpr int kOperandBytes = 16384;           // one operand, one slab
-constexpr int kStageBytes = 2 * kOperandBytes;  // A then B
-constexpr int kLds = kStages * kStageBytes;     // 128 KB
+constexpr int kAStages = 2, kAStageBytes = 32768;  // A ring: pairs of slabs (256 rows x 128 B)
+constexpr int kBStages = 4, kBStageBytes = 16384;  // B ring: single slabs (32 k rows x 512 B)
+constexpr int kBRing = kAStages * kAStageBytes;    // byte offset of the B ring
+constexpr int kRingBytes = kBRing + kBStages * kBStageBytes;  // 128 KB
+constexpr int kStagingBytes = kBM * (kBN * 2 + 16);            // output tile staged for the row-wise store
+constexpr int kLds = kStagingBytes > kRingBytes ? kStagingBytes : kRingBytes;
 constexpr int kXcds = 8;
 
 static_assert(kBM == kRowTile, "row tiles of the schedule must match the GEMM tile");
@@ -91,29 +93,19 @@ __device__ inline u32x2 lds_read_tr16(const char *p) {
   return __builtin_bit_cast(u32x2, v);
 }
 
-// Wait until at most `newer` slabs' worth of this wave's copies (8 each) are still in flight.
-__device__ inline void wait_copies(int newer) {
-  switch (newer) {
-    case 4: asm volatile("s_waitcnt vmcnt(32)" ::: "memory"); break;
-    case 3: asm volatile("s_waitcnt vmcnt(24)" ::: "memory"); break;
-    case 2: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
-    case 1: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
-    default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
-  }
-}
-
 struct TileInfo {
   int expert, row0, rows_valid, n0;
 };
 
 template <typename T, int EPI, int NMI>
-__device__ inline void run_tile(const Args &args, const TileInfo &ti, const char *a_base, const uint32_t (&a_off)[4],
+__device__ inline void run_tile(const Args &args, const TileInfo &ti, const char *a_base, const uint32_t (&a_off)[8],
                                 const char *b_base, const uint32_t (&b_off)[4], long long b_ld_bytes) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in a scalar register
   const int wm = wave >> 1, wn = wave & 1;
   constexpr int NACC = NMI > 0 ? NMI : 1;
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  const uint32_t lds0 = (uint32_t)(uintptr_t)lds;  // LDS byte address of the first slab buffer
+  const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds);  // LDS byte address of the A ring
 
   f32x16 acc[NACC][4];
 #pragma unroll
@@ -123,30 +115,33 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const char
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
 
-  const int n_slabs = args.Kd / kBK;
+  const int n_slabs = args.Kd / kBK;  // even: the contraction length is a multiple of 64
 
   // ---- copy issue ----------------------------------------------------------------------------------
-  // A: this wave fills rows 64*wave + 16*i + (lane >> 2); B: k rows 8*wave + 2*i + (lane >> 5).
-  auto issue = [&](int slab) {
-    const uint32_t stage = lds0 + (uint32_t)(slab % kStages) * kStageBytes;
-    const char *ab = a_base + (long long)slab * (kBK * (int)sizeof(T));
+  // A pair p (slabs 2p, 2p+1): this wave fills rows 64*wave + 8*i + (lane >> 3), 128 bytes each.
+  auto issue_a = [&](int pair) {
+    const uint32_t stage = lds0 + (uint32_t)(pair & (kAStages - 1)) * kAStageBytes;
+    const char *ab = a_base + (long long)pair * (2 * kBK * (int)sizeof(T));
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      copy16_to_lds(ab, a_off[i], stage + (uint32_t)(64 * wave + 8 * i) * 128u);
+  };
+  // B slab: this wave fills k rows 8*wave + 2*i + (lane >> 5), 512 bytes each.
+  auto issue_b = [&](int slab) {
+    const uint32_t stage = lds0 + kBRing + (uint32_t)(slab & (kBStages - 1)) * kBStageBytes;
     const char *bb = b_base + (long long)slab * kBK * b_ld_bytes;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      copy16_to_lds(ab, a_off[i], __builtin_amdgcn_readfirstlane(stage + (uint32_t)(64 * wave + 16 * i) * 64u));
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      copy16_to_lds(bb, b_off[i],
-                    __builtin_amdgcn_readfirstlane(stage + kOperandBytes + (uint32_t)(8 * wave + 2 * i) * 512u));
+      copy16_to_lds(bb, b_off[i], stage + (uint32_t)(8 * wave + 2 * i) * 512u);
   };
 
   // ---- MFMA operand reads ----------------------------------------------------------------------------
-  // A operand (block mi, k-step ks): row (mi*2+wm)*32 + lane%32, piece ks*2 + lane/32.
+  // A operand (block mi, slab parity par, k-step ks): row (mi*2+wm)*32 + lane%32, piece par*4 + ks*2 + lane/32
+  // at position piece ^ ((row >> 1) & 7).
   const int rl = lane & 31, g = lane >> 5;
   int a_rd[2];
 #pragma unroll
-  for (int ks = 0; ks < 2; ++ks)
-    a_rd[ks] = (wm * 32 + rl) * 64 + (((ks * 2 + g) ^ ((rl >> 2) & 3)) << 4);
+  for (int ks = 0; ks < 2; ++ks) a_rd[ks] = (wm * 32 + rl) * 128 + (((ks * 2 + g) ^ ((rl >> 1) & 7)) << 4);
   // B operand (column block ni, k-step ks, half h): k = ks*16 + g*8 + h*4 + j, 4 columns at
   // wn*128 + ni*32 + 16*((lane>>4)&1) + 4*q, where j = (lane&15)>>2 and q = lane&3.
   const int j4 = (lane & 15) >> 2, q4 = lane & 3;
@@ -155,19 +150,23 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const char
   for (int ni = 0; ni < 4; ++ni) {
     int col = wn * 128 + ni * 32 + 16 * ((lane >> 4) & 1) + 4 * q4;
     int piece = (col >> 3) ^ (j4 << 2);
-    b_rd[ni] = kOperandBytes + (g * 8 + j4) * 512 + (piece << 4) + (col & 7) * 2;
+    b_rd[ni] = (g * 8 + j4) * 512 + (piece << 4) + (col & 7) * 2;
   }
 
   u32x4 fa0[NACC], fa1[NACC], fb0[4], fb1[4];
-  auto read_frags = [&](const char *stage, int ks, u32x4 (&fa)[NACC], u32x4 (&fb)[4]) {
+  // slab s: A pair buffer (s>>1)&1, piece offset 64 bytes (XOR) for the odd slab of the pair
+  auto read_frags = [&](int s, int ks, u32x4 (&fa)[NACC], u32x4 (&fb)[4]) {
+    const char *sb = lds + kBRing + (s & (kBStages - 1)) * kBStageBytes;
+    const char *sa = lds + ((s >> 1) & (kAStages - 1)) * kAStageBytes;
+    const int a_o = a_rd[ks] ^ ((s & 1) << 6);
 #pragma unroll
     for (int ni = 0; ni < 4; ++ni) {
-      u32x2 lo = lds_read_tr16(stage + b_rd[ni] + ks * 8192);
-      u32x2 hi = lds_read_tr16(stage + b_rd[ni] + ks * 8192 + 2048);
+      u32x2 lo = lds_read_tr16(sb + b_rd[ni] + ks * 8192);
+      u32x2 hi = lds_read_tr16(sb + b_rd[ni] + ks * 8192 + 2048);
       fb[ni] = (u32x4){lo[0], lo[1], hi[0], hi[1]};
     }
 #pragma unroll
-    for (int mi = 0; mi < NMI; ++mi) fa[mi] = *(const u32x4 *)(stage + a_rd[ks] + mi * 4096);
+    for (int mi = 0; mi < NMI; ++mi) fa[mi] = *(const u32x4 *)(sa + a_o + mi * 8192);
   };
   auto mma = [&](const u32x4 (&fa)[NACC], const u32x4 (&fb)[4]) {
 #pragma unroll
@@ -177,73 +176,108 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const char
   };
 
   // ---- pipeline -----------------------------------------------------------------------------------------
-  const int n_pro = n_slabs < kStages ? n_slabs : kStages;
-  for (int d = 0; d < n_pro; ++d) issue(d);
-  wait_copies(n_pro - 1);
+  // Copy groups are issued after the mid-slab barrier of slab t:  B slab t+4 (4 copies) and, for odd t,
+  // A pair (t+1)/2 + 1 (8 copies).  Copies retire in order, so "slab s+1 has landed" is a bound on how
+  // many younger copies may still be in flight: 4 for odd s, 16 for even s.
+  issue_b(0);
+  issue_a(0);
+  if (n_slabs > 1) issue_b(1);
+  if (n_slabs > 2) { issue_b(2); issue_a(1); }
+  if (n_slabs > 3) issue_b(3);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  read_frags(lds, 0, fa0, fb0);
+  read_frags(0, 0, fa0, fb0);
 
-  for (int s = 0; s < n_slabs; ++s) {
-    const char *stage = lds + (s % kStages) * kStageBytes;
-    const char *next_stage = lds + ((s + 1) % kStages) * kStageBytes;
-    read_frags(stage, 1, fa1, fb1);
+  // One slab: the second k-step's operands are read while the first k-step's MFMAs run; the barrier
+  // sits between the two MFMA groups, followed by the copy issue and the next slab's first reads.
+  auto slab_step = [&](int s, bool odd, bool steady) {
+    read_frags(s, 1, fa1, fb1);
     mma(fa0, fb0);
-    __builtin_amdgcn_sched_barrier(0);
-    if (s + 1 < n_slabs) {
-      int last = n_slabs - 1 < s + kStages - 1 ? n_slabs - 1 : s + kStages - 1;
-      wait_copies(last - (s + 1));  // slab s+1 has landed (this wave's share)
+    if (steady) {
+      if (odd) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
-    // The barrier waits for this wave's LDS reads first, so after it nobody reads slab s's buffer any
+    // The barrier waits for this wave's LDS reads first, so after it nobody reads slab s's buffers any
     // more and everybody's share of slab s+1 is visible.
     __syncthreads();
-    if (s + kStages < n_slabs) issue(s + kStages);
-    if (s + 1 < n_slabs) read_frags(next_stage, 0, fa0, fb0);
+    if (steady || s + kBStages < n_slabs) issue_b(s + kBStages);
+    if (odd && (steady || s + 3 < n_slabs)) issue_a((s + 1) / 2 + 1);
+    if (steady || s + 1 < n_slabs) read_frags(s + 1, 0, fa0, fb0);
     mma(fa1, fb1);
-    __builtin_amdgcn_sched_barrier(0);
+  };
+  int s = 0;
+  for (; s + 7 < n_slabs; s += 2) {  // steady state: every copy group exists
+    slab_step(s, false, true);
+    slab_step(s + 1, true, true);
+  }
+  for (; s < n_slabs; s += 2) {
+    slab_step(s, false, false);
+    slab_step(s + 1, true, false);
   }
 
-  if constexpr (NMI == 0) return;
-
   // ---- epilogue -------------------------------------------------------------------------------------
+  // The output tile is staged in LDS (the slab ring is dead by now) as [row][column] and then written
+  // out row by row with 16 bytes per lane, so that a wave stores whole 512-byte (or 256-byte) row
+  // segments instead of 2 bytes per lane.
   // acc[mi][ni][v]: tile row (mi*2+wm)*32 + 8*(v/4) + 4*(lane/32) + v%4, tile column wn*128 + ni*32 + lane%32
   const int rsub = g * 4;
   const int expert = ti.expert, rows_valid = ti.rows_valid, n0 = ti.n0;
   const long long out_row0 = ti.row0;
-  const bool full = rows_valid == kBM && n0 + kBN <= args.Nd;
-  if constexpr (EPI == EPI_STORE) {
-    T *C = (T *)args.C;
+
+  // rows of `width` elements, row stride width*2 + 16 bytes (the pad spreads the 2-byte stores of the
+  // two lane halves over different banks)
+  auto store_rows = [&](T *dst, long long ld, int col0, int width, int col_limit) {
+    const int stride = width * 2 + 16;
+    const int chunks = width >> 3, rows_per_pass = kThreads / chunks;
+    const int c = tid % chunks;
+    if (col0 + c * 8 >= col_limit) return;
+    T *p = dst + out_row0 * ld + col0 + c * 8;
+    for (int r = tid / chunks; r < rows_valid; r += rows_per_pass)
+      *(u32x4 *)(p + (long long)r * ld) = *(const u32x4 *)(lds + r * stride + c * 16);
+  };
+  // natural column order: value = acc + bias[column]   (the plain product, or the pre-activations)
+  auto stage_biased = [&]() {
+    constexpr int stride = kBN * 2 + 16;
 #pragma unroll
     for (int ni = 0; ni < 4; ++ni) {
-      int col = n0 + wn * 128 + ni * 32 + rl;
-      bool col_ok = col < args.Nd;
+      int lc = wn * 128 + ni * 32 + rl;
       float bias = 0.0f;
-      if (args.bias != nullptr && col_ok)
-        bias = ElemTraits<T>::to_f32(((const T *)args.bias)[(long long)expert * args.Nd + col]);
+      if (args.bias != nullptr && n0 + lc < args.Nd)
+        bias = ElemTraits<T>::to_f32(((const T *)args.bias)[(long long)expert * args.Nd + n0 + lc]);
 #pragma unroll
-      for (int mi = 0; mi < NMI; ++mi) {
-        T *Cp = C + (out_row0 + (mi * 2 + wm) * 32 + rsub) * args.ldc + col;
+      for (int mi = 0; mi < NMI; ++mi)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           int r = (mi * 2 + wm) * 32 + 8 * (v >> 2) + rsub + (v & 3);
-          if (full || (col_ok && r < rows_valid))
-            Cp[(long long)(8 * (v >> 2) + (v & 3)) * args.ldc] = ElemTraits<T>::from_f32(acc[mi][ni][v] + bias);
+          *(T *)(lds + r * stride + lc * 2) = ElemTraits<T>::from_f32(acc[mi][ni][v] + bias);
         }
-      }
     }
+  };
+
+  __syncthreads();  // every wave has finished reading the slab ring
+  if constexpr (EPI == EPI_STORE) {
+    stage_biased();
+    __syncthreads();
+    store_rows((T *)args.C, args.ldc, n0, kBN, args.Nd);
   } else {
+    if (args.C2 != nullptr) {  // pre-activations for the backward: the biased product itself
+      stage_biased();
+      __syncthreads();
+      store_rows((T *)args.C2, args.Nd, n0, kBN, args.Nd);
+      __syncthreads();
+    }
     // Even lanes hold gate columns, odd lanes the matching up columns.  For each pair of accumulator
     // rows (v, v+1) the even lane finishes row v and the odd lane row v+1 after one DPP swap.
-    T *C = (T *)args.C;
-    T *P = (T *)args.C2;
+    constexpr int stride = (kBN / 2) * 2 + 16;
     const bool odd = lane & 1;
 #pragma unroll
     for (int ni = 0; ni < 4; ++ni) {
-      int col = n0 + wn * 128 + ni * 32 + (rl & ~1);  // the gate column of this lane's pair
-      int pair = col >> 1;
-      bool col_ok = col + 1 < args.Nd;
+      int lc = wn * 128 + ni * 32 + (rl & ~1);  // tile column of the gate of this lane's pair
       float bg = 0.0f, bu = 0.0f;
-      if (args.bias != nullptr && col_ok) {
-        const T *bp = (const T *)args.bias + (long long)expert * args.Nd + col;
+      if (args.bias != nullptr && n0 + lc + 1 < args.Nd) {
+        const T *bp = (const T *)args.bias + (long long)expert * args.Nd + n0 + lc;
         bg = ElemTraits<T>::to_f32(bp[0]);
         bu = ElemTraits<T>::to_f32(bp[1]);
       }
@@ -258,17 +292,12 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const char
           float G = (odd ? recv : xe) + bg, U = (odd ? xo : recv) + bu;
           int v = 2 * u + (odd ? 1 : 0);
           int r = (mi * 2 + wm) * 32 + 8 * (v >> 2) + rsub + (v & 3);
-          if (full || (col_ok && r < rows_valid)) {
-            long long orow = out_row0 + r;
-            C[orow * args.ldc + pair] = ElemTraits<T>::from_f32(glu_forward(G, U));
-            if (P != nullptr) {
-              P[orow * args.Nd + col] = ElemTraits<T>::from_f32(G);
-              P[orow * args.Nd + col + 1] = ElemTraits<T>::from_f32(U);
-            }
-          }
+          *(T *)(lds + r * stride + (lc >> 1) * 2) = ElemTraits<T>::from_f32(glu_forward(G, U));
         }
       }
     }
+    __syncthreads();
+    store_rows((T *)args.C, args.ldc, n0 >> 1, kBN / 2, args.Nd >> 1);
   }
 }
 
@@ -296,12 +325,12 @@ __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
     ti.n0 = col_tile * kBN;
   }
 
-  // A copies: rows 64*wave + 16*i + (lane >> 2); LDS position lane & 3 holds piece pos ^ ((row >> 2) & 3)
-  uint32_t a_off[4];
+  // A copies: rows 64*wave + 8*i + (lane >> 3); LDS position lane & 7 holds piece pos ^ ((row >> 1) & 7)
+  uint32_t a_off[8];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    int row = 64 * wave + 16 * i + (lane >> 2);
-    int piece = (lane & 3) ^ ((row >> 2) & 3);
+  for (int i = 0; i < 8; ++i) {
+    int row = 64 * wave + 8 * i + (lane >> 3);
+    int piece = (lane & 7) ^ ((row >> 1) & 7);
     int r = min(row, ti.rows_valid - 1);
     long long src = r;
     if (GATHER) src = args.a_rows[ti.row0 + r] / args.a_div;
@@ -356,7 +385,7 @@ static int launch(const Args &args, int max_row_tiles, hipStream_t stream) {
 
 // True when the asynchronous-copy kernels can take this product.
 bool gemm_async_supported(int Kd, int Nd, int lda, int ldb, long long a_span_bytes) {
-  return Kd % async::kBK == 0 && Kd >= async::kBK && Nd % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 &&
+  return Kd % (2 * async::kBK) == 0 && Kd >= 2 * async::kBK && Nd % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 &&
          a_span_bytes < (1ll << 32);
 }
 

@@ -239,34 +239,53 @@ __global__ __launch_bounds__(kRouteThreads) void route_place_kernel(
 }
 
 // ---- work lists ------------------------------------------------------------------------------
-// One wave; experts are walked in order.  Experts with 1..stream_max_rows kept rows go to the
-// streaming list, larger ones are cut into row tiles of kRowTile rows.
-__global__ void build_schedule_kernel(const int *counts, const int *offsets, int N, int E,
-                                      int capacity, int stream_max_rows, int *sched) {
-  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+// One wave; lane l takes experts l, l+64, ...  Experts with 1..stream_max_rows kept rows go to the
+// streaming list, larger ones are cut into row tiles of kRowTile rows.  Both lists stay in expert
+// order: positions come from wave prefix sums.
+__device__ inline int wave_exclusive_scan(int v, int lane, int &total) {
+  int x = v;
+  for (int d = 1; d < kWave; d <<= 1) {
+    int y = __shfl_up(x, d);
+    if (lane >= d) x += y;
+  }
+  total = __shfl(x, kWave - 1);
+  return x - v;
+}
+
+__global__ __launch_bounds__(kWave) void build_schedule_kernel(const int *counts, const int *offsets, int N, int E,
+                                                               int capacity, int stream_max_rows, int *sched) {
+  const int lane = threadIdx.x;
   int *row_tiles = sched + kSchedHeader;
   int *small = row_tiles + 8 * sched_max_row_tiles(N, E);
   int n_tiles = 0, n_small = 0, n_active = 0, n_kept = 0;
-  for (int e = 0; e < E; ++e) {
-    int kept = min(counts[e], capacity);
-    if (kept <= 0) continue;
-    ++n_active;
-    n_kept += kept;
-    int first = offsets[e];
-    if (kept <= stream_max_rows) {
-      int *s = small + 4 * n_small++;
+  for (int base = 0; base < E; base += kWave) {
+    int e = base + lane;
+    int kept = e < E ? min(counts[e], capacity) : 0;
+    if (kept < 0) kept = 0;
+    int first = e < E ? offsets[e] : 0;
+    int is_small = kept > 0 && kept <= stream_max_rows;
+    int tiles = (kept > 0 && !is_small) ? ceil_div(kept, kRowTile) : 0;
+    int tot_small, tot_tiles, tot_active, tot_kept;
+    int pos_small = wave_exclusive_scan(is_small, lane, tot_small);
+    int pos_tiles = wave_exclusive_scan(tiles, lane, tot_tiles);
+    wave_exclusive_scan(kept > 0 ? 1 : 0, lane, tot_active);
+    wave_exclusive_scan(kept, lane, tot_kept);
+    if (is_small) {
+      int *s = small + 4 * (n_small + pos_small);
       s[0] = e; s[1] = first; s[2] = kept; s[3] = 0;
-    } else {
-      int gfirst = n_tiles, gcount = ceil_div(kept, kRowTile);
-      for (int r = 0; r < kept; r += kRowTile) {
-        int *t = row_tiles + 8 * n_tiles++;
-        t[0] = e; t[1] = first + r; t[2] = min(kRowTile, kept - r); t[3] = gfirst; t[4] = gcount;
-        t[5] = 0; t[6] = 0; t[7] = 0;
-      }
     }
+    int gfirst = n_tiles + pos_tiles;
+    for (int t = 0; t < tiles; ++t) {
+      int *w = row_tiles + 8 * (gfirst + t);
+      w[0] = e; w[1] = first + t * kRowTile; w[2] = min(kRowTile, kept - t * kRowTile); w[3] = gfirst; w[4] = tiles;
+      w[5] = 0; w[6] = 0; w[7] = 0;
+    }
+    n_small += tot_small; n_tiles += tot_tiles; n_active += tot_active; n_kept += tot_kept;
   }
-  sched[0] = n_tiles; sched[1] = n_small; sched[2] = n_active; sched[3] = n_kept;
-  sched[4] = 0; sched[5] = 0; sched[6] = 0; sched[7] = 0;
+  if (lane == 0) {
+    sched[0] = n_tiles; sched[1] = n_small; sched[2] = n_active; sched[3] = n_kept;
+    sched[4] = 0; sched[5] = 0; sched[6] = 0; sched[7] = 0;
+  }
 }
 
 }  // namespace yamoe
