@@ -29,9 +29,10 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
-# HBM bytes per launch of the gate_up GEMM from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (see the
-# counter summary under profiles/); None until measured.
-GATE_UP_TRAFFIC_BYTES = None
+# HBM bytes per launch of the gate_up GEMM on the GPT-OSS-20B workload, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this file (profiles/gemm_async_and_stream_gemm_counters.md): 1 068 960 KiB fetched x 2.0
+# (FETCH_SIZE reads half of a 1 GiB copy's bytes on this device) + 97 381 KiB written x 1.0.
+GATE_UP_TRAFFIC_BYTES = 2.289e9
 
 
 def event_time_ms(fn, iters):
@@ -67,6 +68,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 1 GiB device-to-device copy kernel (a known FETCH_SIZE / WRITE_SIZE for counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (the expert layer here is the "
@@ -84,6 +87,13 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)  # 1 GiB
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---------------- GPT-OSS-20B shaped layer ----------------------------------------------------------
     cfg = workloads.CONFIGS["gptoss20b"]
@@ -123,7 +133,7 @@ def main():
     gu_flop = n_rows * 4 * H * I
     gu_tflops = gu_flop / (gu_ms * 1e-3) / 1e12
     dn_tflops = n_rows * 2 * H * I / (dn_ms * 1e-3) / 1e12
-    roofline = dict(bound="mfma", kernel="grouped_gemm_kernel<bf16, gate_up + GLU>", achieved=round(gu_tflops, 2),
+    roofline = dict(bound="mfma", kernel="gemm_async_kernel<bf16, gate_up + clamped SwiGLU>", achieved=round(gu_tflops, 2),
                     peak=PEAK_BF16_TFLOPS, unit="TFLOP/s", frac=round(gu_tflops / PEAK_BF16_TFLOPS, 4),
                     traffic=GATE_UP_TRAFFIC_BYTES, avg_launch_ms=round(gu_ms, 4),
                     down_gemm=dict(achieved=round(dn_tflops, 2), frac=round(dn_tflops / PEAK_BF16_TFLOPS, 4),
