@@ -1,0 +1,99 @@
+"""CPU-side checks of the boundary: the C-ABI library loads and exports every symbol the header
+declares, argument validation rejects bad shapes before anything touches a GPU, and the torch op is
+registered with the reference's schemas."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, "include", "yamoe_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(yamoe_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from yamoe_amd import _cabi
+    lib = _cabi.lib()
+    names = header_symbols()
+    assert len(names) >= 14
+    for n in names:
+        assert hasattr(lib, n), n
+    assert sorted(_cabi.SYMBOLS) == names
+    assert lib.yamoe_abi_version() == 1
+
+
+def test_size_queries_and_validation_need_no_gpu():
+    from yamoe_amd import _cabi
+    lib = _cabi.lib()
+    p = _cabi.Problem(T=4096, K=4, E=32, H=2880, I=2880, capacity=4096, dtype=_cabi.BF16, idx_i64=1, rw_cols=32)
+    fwd = lib.yamoe_experts_workspace_bytes(ctypes.byref(p))
+    bwd = lib.yamoe_experts_backward_workspace_bytes(ctypes.byref(p))
+    n = 4096 * 4
+    assert fwd >= n * 2880 * 2 * 2 and bwd > fwd            # act + y_perm at least
+    assert fwd < 2 * n * 2880 * 2 * 2                       # and nothing padded to [E, C, *]
+    assert lib.yamoe_schedule_bytes(n, 32) % 256 == 0
+    # rejected shapes: H not a multiple of the 16-byte vector, routing weights with a wrong width, bad dtype
+    for bad in (dict(H=2881), dict(rw_cols=7), dict(dtype=9), dict(K=0)):
+        q = _cabi.Problem(**{**{f: getattr(p, f) for f, _ in p._fields_}, **bad})
+        assert lib.yamoe_experts_workspace_bytes(ctypes.byref(q)) == 0
+        assert len(lib.yamoe_last_error()) > 0
+    # yamoe_route rejects too many experts before any launch
+    rc = lib.yamoe_route(None, 1, 0, 100000, 1, None, None, None, None, None, None, 0, None)
+    assert rc == -1 and b"yamoe_route" in lib.yamoe_last_error()
+    # entry points refuse null pointers instead of launching
+    rc = lib.yamoe_experts_forward(ctypes.byref(p), *([None] * 9), 0, None)
+    assert rc == -1
+
+
+def test_torch_op_schemas_match_reference():
+    import yamoe_amd  # noqa: F401
+    s = str(torch.ops._yamoe_amd_ops.experts.default._schema)
+    assert s == ("_yamoe_amd_ops::experts(Tensor hidden_states, Tensor router_indices, Tensor routing_weights, "
+                 "Tensor gate_up_proj, Tensor gate_up_proj_bias, Tensor down_proj, Tensor down_proj_bias, "
+                 "int expert_capacity, int num_experts, int top_k) -> Tensor")
+    s = str(torch.ops._yamoe_amd_ops.experts_backward.default._schema)
+    assert s.startswith("_yamoe_amd_ops::experts_backward(Tensor grad_out, Tensor hidden_states, Tensor router_indices, ")
+    assert s.endswith("int expert_capacity, int num_experts, int top_k) -> Tensor[]")
+
+
+def test_no_cpu_fallback():
+    """CPU tensors are refused: there is no eager or oracle path behind the op."""
+    import yamoe_amd
+    from yamoe_amd import _cabi
+    from yamoe_amd.workloads import make_inputs
+    d = make_inputs(8, 64, 64, 4, 2, torch.float32)
+    a = [d[k] for k in ("hidden", "router_indices", "routing_weights", "gate_up_proj", "gate_up_proj_bias",
+                        "down_proj", "down_proj_bias")]
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        yamoe_amd.experts(*a, 8, 4, 2)
+    with pytest.raises(RuntimeError):
+        _cabi.experts_forward(*a, 8)
+
+
+def test_product_does_not_import_the_oracle():
+    for dirpath, _, files in os.walk(os.path.join(ROOT, "yamoe_amd")):
+        for f in files:
+            if f.endswith((".py", ".hip", ".cpp", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.replace("no oracle", ""), os.path.join(dirpath, f)
+
+
+def test_workloads_are_seeded_and_shaped():
+    from yamoe_amd.workloads import CONFIGS, make_config
+    a, c = make_config("decode", seed=3, weights=False)
+    b, _ = make_config("decode", seed=3, weights=False)
+    assert torch.equal(a["router_indices"], b["router_indices"]) and torch.equal(a["hidden"], b["hidden"])
+    assert a["router_indices"].shape == (64, 4) and a["routing_weights"].shape == (64, 128)
+    rw = a["routing_weights"].float()
+    assert torch.allclose(rw.sum(1), torch.ones(64), atol=2e-2)  # renormalised top-4 (bf16 rounding)
+    assert (rw > 0).sum(1).eq(4).all()
+    z, _ = make_config("zipf", seed=0, weights=False)
+    counts = torch.bincount(z["router_indices"].flatten(), minlength=128)
+    assert counts.max() > 10 * counts.float().mean() and (counts == 0).any()
+    assert set(CONFIGS) == {"readme", "gptoss20b", "decode", "zipf"}
