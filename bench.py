@@ -68,6 +68,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--extras", action="store_true",
+                    help="also time the backward (GPT-OSS-20B shape), the Zipf-skewed and the README fp32 workloads")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy kernel (a known FETCH_SIZE / WRITE_SIZE for counter runs)")
     args = ap.parse_args()
@@ -193,6 +195,55 @@ def main():
                       algorithmic_bytes=nbytes,
                       config=dict(workload="decode: T=64 H=I=2880 E=128 top-4 bf16", tokens=Td, experts=Ed, top_k=Kd))
 
+    extras = None
+    if args.extras:
+        extras = {}
+        try:
+            del dd, ad
+        except NameError:
+            del d, a, act, y
+        torch.cuda.empty_cache()
+
+        def timed(fn, n_flop, label, iters=max(3, args.steps // 4)):
+            for _ in range(2):
+                fn()
+            ms = event_time_ms(fn, iters)
+            extras[label] = dict(ms=round(ms, 4), tflops=round(n_flop / (ms * 1e-3) / 1e12, 2),
+                                 frac_of_peak=round(n_flop / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4))
+
+        # backward at the GPT-OSS-20B shape: 18*H*I flop per assignment (forward recompute + dgrad + wgrad)
+        hostb, _ = workloads.make_config("gptoss20b", seed=0, weights=False)
+        db = {k: v.to(dev) for k, v in hostb.items()}
+        db.update(device_weights(E, H, I, torch.bfloat16, cfg["w_std"], 1, dev))
+        ab = [db[k] for k in order]
+        gy = torch.randn(T, H, device=dev, generator=torch.Generator(device=dev).manual_seed(3)).to(torch.bfloat16)
+        timed(lambda: yamoe_amd.experts_backward(gy, *ab, T, E, K), T * K * 18 * H * I, "backward_gptoss20b_bf16")
+        del db, ab, gy
+        torch.cuda.empty_cache()
+        # Zipf-skewed routing, 16384 tokens, 128 experts
+        zc = workloads.CONFIGS["zipf"]
+        hostz, _ = workloads.make_config("zipf", seed=0, weights=False)
+        dz = {k: v.to(dev) for k, v in hostz.items()}
+        dz.update(device_weights(zc["E"], H, I, torch.bfloat16, zc["w_std"], 4, dev))
+        az = [dz[k] for k in order]
+        timed(lambda: yamoe_amd.experts(*az, zc["T"], zc["E"], zc["K"]), zc["T"] * zc["K"] * 6 * H * I,
+              "forward_zipf_bf16")
+        cz = np.bincount(hostz["router_indices"].numpy().ravel(), minlength=zc["E"])
+        extras["forward_zipf_bf16"].update(max_rows=int(cz.max()), empty_experts=int((cz == 0).sum()))
+        del dz, az
+        torch.cuda.empty_cache()
+        # README shape, fp32 (peak 157.3 TFLOP/s fp32 MFMA)
+        rc = workloads.CONFIGS["readme"]
+        hostr, _ = workloads.make_config("readme", seed=42, weights=False)
+        dr = {k: v.to(dev) for k, v in hostr.items()}
+        dr.update(device_weights(rc["E"], H, I, torch.float32, 1.0, 5, dev))
+        dr["gate_up_proj_bias"].zero_()
+        dr["down_proj_bias"].zero_()
+        ar = [dr[k] for k in order]
+        timed(lambda: yamoe_amd.experts(*ar, rc["T"], rc["E"], rc["K"]), rc["T"] * rc["K"] * 6 * H * I,
+              "forward_readme_fp32")
+        extras["forward_readme_fp32"]["frac_of_peak"] = round(extras["forward_readme_fp32"]["tflops"] / 157.3, 4)
+
     line = dict(metric="experts_fwd_tflops", value=round(value, 2), unit="TFLOP/s", n_gpus=1, steps=args.steps,
                 warmup=args.warmup, ms_per_step=round(ms_per_step, 4), higher_is_better=True, scaling="weak",
                 vs_baseline=None, dtype="bf16", data="synthetic",
@@ -200,7 +251,7 @@ def main():
                             tokens=T, hidden=H, intermediate=I, experts=E, top_k=K,
                             algorithmic_flop=flop),
                 frac_of_mfma_peak=round(value / PEAK_BF16_TFLOPS, 4), roofline=roofline, cpu_baseline=cpu_baseline,
-                parity=parity, decode=decode)
+                parity=parity, decode=decode, extras=extras)
     print(json.dumps(line))
 
 
