@@ -24,7 +24,7 @@ HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall",
     # packed fp32 VALU forms are switched off on purpose (they have produced silent wrong results)
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-]
+] + os.environ.get("YAMOE_HIPCC_EXTRA", "").split()
 
 
 def _run(cmd):

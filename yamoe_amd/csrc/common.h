@@ -56,7 +56,8 @@ __host__ __device__ inline size_t align_up(size_t v, size_t a) { return (v + a -
 __device__ inline float glu_forward(float G, float U) {
   float g = fminf(G, kGluLimit);
   float u = fminf(fmaxf(U, -kGluLimit), kGluLimit);
-  float s = 1.0f / (1.0f + __expf(-kGluAlpha * g));
+  // sigmoid through the hardware exp2 and reciprocal (each about 1 ulp); exp2(+inf) -> s = 0, the right limit
+  float s = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * (-kGluAlpha * 1.44269504088896341f)));
   return (u + 1.0f) * (g * s);
 }
 

@@ -176,9 +176,11 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const char
   };
 
   // ---- pipeline -----------------------------------------------------------------------------------------
-  // Copy groups are issued after the mid-slab barrier of slab t:  B slab t+4 (4 copies) and, for odd t,
-  // A pair (t+1)/2 + 1 (8 copies).  Copies retire in order, so "slab s+1 has landed" is a bound on how
-  // many younger copies may still be in flight: 4 for odd s, 16 for even s.
+  // Copy groups are issued after the mid-slab barrier of slab t: for odd t the A pair (t+1)/2 + 1
+  // (8 copies), then B slab t+4 (4 copies).  Copies retire in order and the A pair is needed two slabs
+  // later while the B slab has four, so A goes first: a weight fetch that misses to HBM then never
+  // delays an activation fetch that hits in L2.  "Slab s+1 has landed" is a bound on how many younger
+  // copies may still be in flight: 8 for odd s, 16 for even s.
   issue_b(0);
   issue_a(0);
   if (n_slabs > 1) issue_b(1);
@@ -194,7 +196,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const char
     read_frags(s, 1, fa1, fb1);
     mma(fa0, fb0);
     if (steady) {
-      if (odd) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      if (odd) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
       else asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
     } else {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -202,8 +204,8 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const char
     // The barrier waits for this wave's LDS reads first, so after it nobody reads slab s's buffers any
     // more and everybody's share of slab s+1 is visible.
     __syncthreads();
-    if (steady || s + kBStages < n_slabs) issue_b(s + kBStages);
     if (odd && (steady || s + 3 < n_slabs)) issue_a((s + 1) / 2 + 1);
+    if (steady || s + kBStages < n_slabs) issue_b(s + kBStages);
     if (steady || s + 1 < n_slabs) read_frags(s + 1, 0, fa0, fb0);
     mma(fa1, fb1);
   };
