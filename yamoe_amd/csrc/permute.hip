@@ -49,6 +49,10 @@ __device__ inline float slot_weight(const T *rw, const void *idx, int t, int k, 
 }
 
 // out[t,:] = sum_k w(t,k) * y_perm[inv_pos[t*K+k],:]
+// One wave per token.  The K (position, weight) pairs of the token are fetched once (up to kMaxSlots of
+// them sit in registers), then every lane streams its 16-byte chunks of the K rows.
+constexpr int kMaxSlots = 8;
+
 template <typename T, bool I64>
 __global__ __launch_bounds__(kRowThreads) void combine_kernel(
     const T *__restrict__ y_perm, const int *__restrict__ inv_pos, const void *__restrict__ idx,
@@ -60,19 +64,29 @@ __global__ __launch_bounds__(kRowThreads) void combine_kernel(
   const bool vec_ok = (H % V) == 0;
   for (int t = wave; t < Tn; t += n_waves) {
     T *dst = out + (size_t)t * H;
-    if (vec_ok) {
+    if (vec_ok && K <= kMaxSlots) {
+      int pos[kMaxSlots];
+      float w[kMaxSlots];
+#pragma unroll
+      for (int k = 0; k < kMaxSlots; ++k) {
+        pos[k] = -1;
+        w[k] = 0.0f;
+        if (k < K) {
+          pos[k] = inv_pos[(size_t)t * K + k];
+          if (pos[k] >= 0) w[k] = slot_weight<T, I64>(rw, idx, t, k, K, E, rw_cols);
+        }
+      }
       for (int c = lane; c < H / V; c += kWave) {
         float acc[V];
 #pragma unroll
         for (int j = 0; j < V; ++j) acc[j] = 0.0f;
-        for (int k = 0; k < K; ++k) {
-          int pos = inv_pos[(size_t)t * K + k];
-          if (pos < 0) continue;
-          float w = slot_weight<T, I64>(rw, idx, t, k, K, E, rw_cols);
-          u32x4 raw = ((const u32x4 *)(y_perm + (size_t)pos * H))[c];
+#pragma unroll
+        for (int k = 0; k < kMaxSlots; ++k) {
+          if (pos[k] < 0) continue;
+          u32x4 raw = ((const u32x4 *)(y_perm + (size_t)pos[k] * H))[c];
           const T *v = (const T *)&raw;
 #pragma unroll
-          for (int j = 0; j < V; ++j) acc[j] += w * ElemTraits<T>::to_f32(v[j]);
+          for (int j = 0; j < V; ++j) acc[j] += w[k] * ElemTraits<T>::to_f32(v[j]);
         }
         u32x4 o;
         T *ov = (T *)&o;

@@ -66,10 +66,20 @@ __device__ inline void wave_place(const void *idx, int seg_begin, int seg_end, i
   const int lane = threadIdx.x & (kWave - 1);
   const int key_bits = bits_for(E + 1);
   const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  // the raw id of the next step is fetched one step ahead so that its latency hides behind this step
+  int raw_next = (seg_begin + lane < seg_end) ? load_raw<I64>(idx, seg_begin + lane) : 0;
+  bool bad_next = (seg_begin + lane < seg_end) ? (load_key<I64>(idx, seg_begin + lane, E) == E) : false;
   for (int base = seg_begin; base < seg_end; base += kWave) {
     int i = base + lane;
     bool active = i < seg_end;
-    int key = active ? load_key<I64>(idx, i, E) : 0;
+    int raw = raw_next;
+    int key = bad_next ? E : raw;
+    if (!active) key = 0;
+    int in = i + kWave;
+    if (in < seg_end) {
+      raw_next = load_raw<I64>(idx, in);
+      bad_next = load_key<I64>(idx, in, E) == E;
+    }
     uint64_t peers = match_key(key, active, key_bits);
     int rank = __popcll(peers & lt_mask);
     int start = 0;
@@ -77,7 +87,7 @@ __device__ inline void wave_place(const void *idx, int seg_begin, int seg_end, i
     __builtin_amdgcn_wave_barrier();
     if (active) {
       int pos = start + rank;
-      sorted_expert[pos] = load_raw<I64>(idx, i);
+      sorted_expert[pos] = raw;
       sorted_idx[pos] = i;
       bool kept = key < E && (pos - offsets_lds[key]) < capacity;
       inv_pos[i] = kept ? pos : -1;
