@@ -134,6 +134,52 @@ int yamoe_experts_backward(const yamoe_problem *p, const void *grad_out,
                            void *d_down_proj_bias, void *workspace, size_t workspace_bytes,
                            void *stream);
 
+/* ---- helper ops on the reference's own layouts (torch-ext/torch_binding.cpp:9-56) ---------
+ * These serve code written against the reference's public helper ops; the fused forward and
+ * backward above do not use them. */
+
+/* sort_cuda (csrc/sort.cu:61-91): stable radix sort of int16/int32/int64 keys on bits
+ * [0, end_bit), payload = iota of the key type.  elem_bytes = 2, 4 or 8. */
+size_t yamoe_sort_workspace_bytes(int32_t n, int32_t elem_bytes);
+int yamoe_sort(const void *x, int32_t elem_bytes, int32_t n, int32_t end_bit, void *x_out,
+               void *iota_out, void *workspace, size_t workspace_bytes, void *stream);
+
+/* bincount_cumsum_cuda (csrc/bincount_cumsum.cu:58-97): output[b] = number of inputs <= b for
+ * b < minlength (inclusive prefix sum of the bin counts); output[minlength..output_len) = 0. */
+int yamoe_bincount_cumsum(const int32_t *input, int32_t n, int32_t *output, int32_t output_len,
+                          int32_t minlength, void *stream);
+
+/* gather_cuda (csrc/gather.cu:68-109): output[e,i,:] = x[indices[start_e+i] / top_k,:] for
+ * i < bins[e]-start_e (start_e = bins[e-1], inclusive bins), zero elsewhere; output is [E,C,H]. */
+int yamoe_padded_gather(const void *x, const int32_t *indices, const int32_t *bins, void *output,
+                        int32_t T, int32_t H, int32_t E, int32_t C, int32_t top_k, int32_t dtype,
+                        void *stream);
+
+/* scatter_cuda (csrc/scatter.cu:110-147): y[tok,:] += src[e,i,:] * weights[start_e+i] for the
+ * first C rows of every expert; weights == NULL means 1.  No atomics: fp32 sum per output row in
+ * slot order on top of the incoming y. */
+size_t yamoe_padded_scatter_workspace_bytes(int32_t S);
+int yamoe_padded_scatter(const void *src, const int32_t *indices, const int32_t *bins,
+                         const void *weights, void *y, int32_t T, int32_t H, int32_t E, int32_t C,
+                         int32_t top_k, int32_t dtype, void *workspace, size_t workspace_bytes,
+                         void *stream);
+
+/* index_select_out_cuda (csrc/index_select.cu:18-51): out[i] = input[idx[i]]. */
+int yamoe_index_select(const void *input, const int32_t *idx, void *out, int64_t n, int32_t dtype,
+                       void *stream);
+
+/* counts[e] = rows, offsets[e] = e*rows (offsets has E+1 entries): the regular [E,rows,*] layout
+ * described as ragged groups, used by yamoe_batch_mm. */
+int yamoe_regular_groups(int32_t *counts, int32_t *offsets, int32_t E, int32_t rows, void *stream);
+
+/* batch_mm (csrc/batch_mm.cu:7-31): output[e] = x[e] . weights[e] for x [E,C,Kd], weights
+ * [E,Kd,Nd], output [E,C,Nd], on the grouped MFMA / streaming kernels.  Like the reference,
+ * every one of the C rows is computed (batch_sizes is not consulted). */
+size_t yamoe_batch_mm_workspace_bytes(int32_t E, int32_t C);
+int yamoe_batch_mm(const void *x, const void *weights, void *output, int32_t E, int32_t C,
+                   int32_t Kd, int32_t Nd, int32_t dtype, void *workspace, size_t workspace_bytes,
+                   void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -22,6 +22,15 @@ formula under test):
                         capacity >= max load
   experts_backward      torch.autograd.gradcheck of experts_capacity in fp64 (finite differences),
                         and agreement between autograd and the closed-form experts_backward_closed
+  sort_pairs            numpy's stable argsort on the masked key (a library routine), order and
+                        stability invariants, two's-complement cases worked by hand
+  bincount_cumsum       numpy bincount + cumsum (library), last entry = number of in-range items
+  padded_gather / padded_scatter / batch_mm / index_select
+                        composed as sort -> bincount_cumsum -> gather -> batch_mm -> glu -> batch_mm
+                        -> scatter (the pipeline of torch-ext/yamoe/vendored/yamoe_ref.py:31-70) they
+                        must reproduce experts_capacity, which is pinned on its own above; padding
+                        rows must be zero; gather followed by unweighted scatter multiplies each
+                        token row by its number of kept slots
 The reference ships no golden vectors or known-answer tests for this path (its tests directory is
 git-ignored), so no reference-held fixture exists to check against; no function here is
 "parity unpinned" in the sense of lacking an independent check.
@@ -231,6 +240,79 @@ def experts_backward_closed(grad_out, hidden, router_indices, routing_weights, g
 # ------------------------------------------------------------------------------------------------
 # metrics (definitions of compare_example.py:207-214)
 # ------------------------------------------------------------------------------------------------
+# ------------------------------------------------------------------------------------------------
+# helper ops on the padded [E, C, H] layout
+# ------------------------------------------------------------------------------------------------
+def sort_pairs(x, end_bit):
+    """Stable sort of integer keys on their low `end_bit` bits, carrying positions
+    (csrc/sort.cu:17-91: cub::DeviceRadixSort::SortPairs with begin_bit 0, an arange payload of the
+    keys' dtype).  With end_bit equal to the key width the order is the signed order (the radix sort
+    flips the sign bit of signed keys); with fewer bits the sign bit takes no part and the order is
+    that of the unsigned low bits.  Returns (sorted keys, positions cast to the key dtype)."""
+    x = np.asarray(x)
+    width = x.dtype.itemsize * 8
+    assert 0 <= end_bit <= width
+    u = x.astype(np.int64).view(np.uint64) & np.uint64((1 << width) - 1 if width < 64 else 0xFFFFFFFFFFFFFFFF)
+    if end_bit == width:
+        key = u ^ np.uint64(1 << (width - 1))
+    else:
+        key = u & np.uint64((1 << end_bit) - 1)
+    perm = np.argsort(key, kind="stable")
+    return x[perm], perm.astype(x.dtype)
+
+
+def bincount_cumsum(values, out_len, minlength):
+    """Inclusive running total of the histogram of `values` over [0, minlength); entries out of
+    range are ignored and the rest of the output is zero (csrc/bincount_cumsum.cu:7-97)."""
+    v = np.asarray(values).astype(np.int64)
+    v = v[(v >= 0) & (v < minlength)]
+    out = np.zeros(out_len, dtype=np.int32)
+    out[:minlength] = np.cumsum(np.bincount(v, minlength=minlength)[:minlength])
+    return out
+
+
+def padded_gather(x, indices, bins, E, C, top_k):
+    """out[e, i] = x[indices[start_e + i] // top_k] for i < bins[e] - start_e, else zero
+    (csrc/gather.cu:6-61); start_e = bins[e-1], start_0 = 0."""
+    T, H = x.shape
+    out = torch.zeros(E, C, H, dtype=x.dtype)
+    for e in range(E):
+        start = 0 if e == 0 else int(bins[e - 1])
+        n = int(bins[e]) - start
+        for i in range(min(n, C)):
+            tok = int(indices[start + i]) // top_k
+            if 0 <= tok < T:
+                out[e, i] = x[tok]
+    return out
+
+
+def padded_scatter(src, indices, bins, weights, y, T, E, C, top_k, compute_dtype=torch.float64):
+    """y[indices[start_e + i] // top_k] += src[e, i] * weights[start_e + i] over the same rows as
+    padded_gather (csrc/scatter.cu:66-105); weights are in sorted order, None means 1.  Accumulated
+    in `compute_dtype` on top of y's content and returned in that dtype."""
+    acc = y.to(compute_dtype).clone()
+    for e in range(E):
+        start = 0 if e == 0 else int(bins[e - 1])
+        n = int(bins[e]) - start
+        for i in range(min(n, C)):
+            tok = int(indices[start + i]) // top_k
+            if 0 <= tok < T:
+                w = 1.0 if weights is None else weights[start + i].to(compute_dtype)
+                acc[tok] += src[e, i].to(compute_dtype) * w
+    return acc
+
+
+def index_select(values, idx):
+    """out[i] = values[idx[i]] on flat tensors (csrc/index_select.cu:7-16)."""
+    return values.reshape(-1)[idx.to(torch.int64)]
+
+
+def batch_mm(x, weights, compute_dtype=torch.float64):
+    """Per-expert product [E, C, K] x [E, K, N]; batch_sizes and trans_b are not used by the
+    reference (csrc/batch_mm.cu:7-31 is one bmm)."""
+    return torch.bmm(x.to(compute_dtype), weights.to(compute_dtype))
+
+
 def rel_l2(a, b):
     a, b = a.double().cpu(), b.double().cpu()
     return float((a - b).norm() / b.norm().clamp_min(1e-30))

@@ -224,3 +224,75 @@ def test_backward_routing_grad_is_zero_outside_selection():
     sel = torch.zeros_like(d_rw, dtype=torch.bool).scatter_(1, d["router_indices"], True)
     assert torch.all(d_rw[~sel] == 0)
     assert torch.any(d_rw[sel] != 0)
+
+
+# ---- helper ops on the padded layout ---------------------------------------------------------------------
+def test_sort_pairs_two_complement_cases_by_hand():
+    x = np.array([3, -1, 0, -128, 3, 127], dtype=np.int16)
+    k, p = O.sort_pairs(x, 16)                  # full width: signed order, ties in input order
+    assert k.tolist() == [-128, -1, 0, 3, 3, 127] and p.tolist() == [3, 1, 2, 0, 4, 5]
+    # low 3 bits only: 3->3, -1->7, 0->0, -128->0, 3->3, 127->7
+    k, p = O.sort_pairs(x, 3)
+    assert p.tolist() == [2, 3, 0, 4, 1, 5] and k.tolist() == [0, -128, 3, 3, -1, 127]
+    k, p = O.sort_pairs(x, 0)                   # no bits: nothing moves
+    assert p.tolist() == [0, 1, 2, 3, 4, 5]
+
+
+@pytest.mark.parametrize("dt", [np.int16, np.int32, np.int64])
+def test_sort_pairs_invariants(dt):
+    rng = np.random.default_rng(5)
+    info = np.iinfo(dt)
+    x = rng.integers(info.min, info.max, size=3000, dtype=dt, endpoint=True)
+    x[:50] = x[50:100]                           # ties
+    k, p = O.sort_pairs(x, info.bits)
+    assert np.all(np.diff(k.astype(object)) >= 0)
+    assert np.array_equal(x[p.astype(np.int64)], k) and np.array_equal(k, np.sort(x))
+    same = k[1:] == k[:-1]
+    assert np.all(p[1:][same] > p[:-1][same])    # stable
+
+
+def test_bincount_cumsum_by_hand():
+    out = O.bincount_cumsum([2, 0, 2, 5, -1, 2, 9], out_len=8, minlength=6)
+    assert out.tolist() == [1, 1, 4, 4, 4, 5, 0, 0]
+
+
+@pytest.mark.parametrize("C", [3, 64])
+def test_padded_helpers_compose_to_the_expert_op(C):
+    """sort -> bincount_cumsum -> gather -> batch_mm -> glu -> batch_mm -> scatter is the reference's
+    own composition (torch-ext/yamoe/vendored/yamoe_ref.py:31-70) and must give the op's result."""
+    d = tiny(seed=4, T=40, E=5, K=3)
+    T, K = d["router_indices"].shape
+    E, H = 5, d["hidden"].shape[1]
+    flat = d["router_indices"].reshape(-1).numpy().astype(np.int32)
+    keys, pos = O.sort_pairs(flat, 32)
+    bins = O.bincount_cumsum(keys, E, E)
+    x = O.padded_gather(d["hidden"], pos, bins, E, C, K)
+    # padding rows are zero
+    for e in range(E):
+        n = bins[e] - (bins[e - 1] if e else 0)
+        assert torch.all(x[e, min(n, C):] == 0)
+    gu = O.batch_mm(x, d["gate_up_proj"]) + d["gate_up_proj_bias"][:, None, :]
+    y = O.batch_mm(O.glu(gu), d["down_proj"]) + d["down_proj_bias"][:, None, :]
+    w_sorted = O.index_select(d["routing_weights"].gather(1, d["router_indices"]).reshape(-1), torch.from_numpy(pos))
+    out = O.padded_scatter(y, pos, bins, w_sorted, torch.zeros(T, H, dtype=torch.float64), T, E, C, K)
+    want = O.experts_capacity(*args(d), C, compute_dtype=torch.float64)
+    assert O.rel_l2(out, want) < 1e-12
+
+
+def test_gather_then_plain_scatter_counts_kept_slots():
+    d = tiny(seed=6, T=30, E=4, K=2)
+    T, K, E, C = 30, 2, 4, 9
+    flat = d["router_indices"].reshape(-1).numpy().astype(np.int32)
+    keys, pos = O.sort_pairs(flat, 32)
+    bins = O.bincount_cumsum(keys, E, E)
+    x = O.padded_gather(d["hidden"], pos, bins, E, C, K)
+    y0 = torch.ones(T, d["hidden"].shape[1], dtype=torch.float64)
+    out = O.padded_scatter(x, pos, bins, None, y0, T, E, C, K)
+    r = O.route(d["router_indices"], E, C)
+    kept = np.zeros(T)
+    for p_sorted, f in enumerate(r["sorted_idx"]):
+        e = r["sorted_expert"][p_sorted]
+        if 0 <= e < E and p_sorted - r["offsets"][e] < C:
+            kept[f // K] += 1
+    want = y0 + d["hidden"] * torch.from_numpy(kept)[:, None]
+    assert O.rel_l2(out, want) < 1e-14

@@ -20,7 +20,9 @@ SYMBOLS = [
     "yamoe_abi_version", "yamoe_last_error", "yamoe_route_workspace_bytes", "yamoe_route", "yamoe_permute",
     "yamoe_combine", "yamoe_schedule_bytes", "yamoe_build_schedule", "yamoe_gate_up", "yamoe_down",
     "yamoe_experts_workspace_bytes", "yamoe_experts_forward", "yamoe_experts_backward_workspace_bytes",
-    "yamoe_experts_backward",
+    "yamoe_experts_backward", "yamoe_sort_workspace_bytes", "yamoe_sort", "yamoe_bincount_cumsum", "yamoe_padded_gather",
+    "yamoe_padded_scatter_workspace_bytes", "yamoe_padded_scatter", "yamoe_index_select", "yamoe_regular_groups",
+    "yamoe_batch_mm_workspace_bytes", "yamoe_batch_mm",
 ]
 
 

@@ -377,3 +377,35 @@ extern "C" int yamoe_experts_backward(const yamoe_problem *p, const void *grad_o
                                             d_gate_up_proj, d_gate_up_proj_bias, d_down_proj, d_down_proj_bias,
                                             workspace, (hipStream_t)stream));
 }
+
+// ---- batch_mm on the regular [E, C, *] layout -------------------------------------------------------
+extern "C" size_t yamoe_batch_mm_workspace_bytes(int32_t E, int32_t C) {
+  if (E <= 0 || C < 0) return 0;
+  return align_up((size_t)E * 4, 256) + align_up(((size_t)E + 1) * 4, 256) + yamoe_schedule_bytes(E * C, E);
+}
+
+template <typename T>
+static int batch_mm_impl(const void *x, const void *w, void *out, int E, int C, int Kd, int Nd, void *ws,
+                         hipStream_t stream) {
+  Carver c(ws);
+  int *counts = (int *)c.take((size_t)E * 4);
+  int *offsets = (int *)c.take(((size_t)E + 1) * 4);
+  size_t sched_bytes = yamoe_schedule_bytes(E * C, E);
+  void *sched = c.take(sched_bytes);
+  YAMOE_TRY(yamoe_regular_groups(counts, offsets, E, C, (void *)stream));
+  const int stream_rows = HasStreamPath<T>::value ? kStreamMaxRows : 0;
+  YAMOE_TRY(yamoe_build_schedule(counts, offsets, E * C, E, C, stream_rows, sched, sched_bytes, (void *)stream));
+  // the down-projection launchers compute rows[.,Kd] x w[e][Kd,Nd] with no bias: exactly this product
+  return down_both<T>(x, w, nullptr, out, sched, E * C, E, /*H=*/Nd, /*I=*/Kd, stream);
+}
+
+extern "C" int yamoe_batch_mm(const void *x, const void *weights, void *output, int32_t E, int32_t C, int32_t Kd,
+                              int32_t Nd, int32_t dtype, void *workspace, size_t workspace_bytes, void *stream) {
+  YAMOE_TRY(check_gemm_shape("yamoe_batch_mm", E * C, E, Nd, Kd, dtype));
+  if (C <= 0) return 0;
+  if (!x || !weights || !output || !workspace || workspace_bytes < yamoe_batch_mm_workspace_bytes(E, C)) {
+    set_error("yamoe_batch_mm: null pointer or workspace too small");
+    return YAMOE_E_ARG;
+  }
+  YAMOE_DISPATCH(dtype, batch_mm_impl<T>(x, weights, output, E, C, Kd, Nd, workspace, (hipStream_t)stream));
+}

@@ -155,9 +155,140 @@ std::vector<at::Tensor> experts_backward(const at::Tensor &grad_out, const at::T
   return {d_hidden, d_routing, d_wgu, d_bgu, d_wd, d_bd};
 }
 
+
+// ---- helper ops on the reference's layouts (torch-ext/torch_binding.cpp:9-56) -----------------------------
+void *current_stream() { return (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream(); }
+
+void check_i32(const at::Tensor &t, const char *name) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kInt && t.is_contiguous(), name, " must be a contiguous int32 GPU tensor");
+}
+
+void gather_op(const at::Tensor &x, const at::Tensor &indices, const at::Tensor &bins, at::Tensor &output, int64_t E,
+               int64_t C, int64_t top_k) {
+  TORCH_CHECK(x.is_cuda() && x.dim() == 2 && x.is_contiguous(), "x must be a contiguous [T, H] GPU tensor");
+  check_i32(indices, "indices");
+  check_i32(bins, "bins");
+  const int64_t T = x.size(0), H = x.size(1);
+  TORCH_CHECK(output.is_cuda() && output.is_contiguous() && output.dim() == 3 && output.size(0) == E &&
+                  output.size(1) == C && output.size(2) == H && output.scalar_type() == x.scalar_type(),
+              "Output tensor must have shape [E, C, H]");
+  TORCH_CHECK(bins.numel() >= E, "bins must have at least E entries");
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+  check_rc(yamoe_padded_gather(x.data_ptr(), indices.data_ptr<int>(), bins.data_ptr<int>(), output.data_ptr(), (int)T,
+                               (int)H, (int)E, (int)C, (int)top_k, dtype_code(x, "x"), current_stream()),
+           "yamoe_padded_gather");
+}
+
+void scatter_op(const at::Tensor &src, const at::Tensor &indices, const at::Tensor &bins, const at::Tensor &weights,
+                at::Tensor &y, int64_t T, int64_t E, int64_t C, int64_t top_k) {
+  TORCH_CHECK(src.is_cuda() && src.dim() == 3 && src.is_contiguous() && src.size(0) == E && src.size(1) == C,
+              "src must be a contiguous [E, C, H] GPU tensor");
+  check_i32(indices, "indices");
+  check_i32(bins, "bins");
+  const int64_t H = src.size(2);
+  TORCH_CHECK(y.is_cuda() && y.is_contiguous() && y.dim() == 2 && y.size(0) == T && y.size(1) == H &&
+                  y.scalar_type() == src.scalar_type(), "y must be a contiguous [T, H] tensor of src's dtype");
+  TORCH_CHECK(indices.numel() == T * top_k, "indices must have T*top_k entries");
+  const void *w = nullptr;
+  if (weights.defined() && weights.numel() > 0) {
+    TORCH_CHECK(weights.is_cuda() && weights.is_contiguous() && weights.scalar_type() == src.scalar_type() &&
+                    weights.numel() == T * top_k, "weights must be [T*top_k] of src's dtype");
+    w = weights.data_ptr();
+  }
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(src.device());
+  size_t ws_bytes = yamoe_padded_scatter_workspace_bytes((int)(T * top_k));
+  at::Tensor ws = at::empty({(int64_t)ws_bytes}, src.options().dtype(at::kByte));
+  check_rc(yamoe_padded_scatter(src.data_ptr(), indices.data_ptr<int>(), bins.data_ptr<int>(), w, y.data_ptr(), (int)T,
+                                (int)H, (int)E, (int)C, (int)top_k, dtype_code(src, "src"), ws.data_ptr(), ws_bytes,
+                                current_stream()),
+           "yamoe_padded_scatter");
+}
+
+void sort_op(at::Tensor x, int64_t end_bit, at::Tensor x_out, at::Tensor iota_out) {
+  TORCH_CHECK(x.is_cuda() && x.dim() == 1, "x must be a 1-D GPU tensor");
+  TORCH_CHECK(x.scalar_type() == at::kShort || x.scalar_type() == at::kInt || x.scalar_type() == at::kLong,
+              "x must be int16, int32 or int64");
+  TORCH_CHECK(x_out.is_cuda() && x_out.dim() == 1 && x_out.scalar_type() == x.scalar_type() && x_out.numel() == x.numel());
+  TORCH_CHECK(iota_out.is_cuda() && iota_out.dim() == 1 && iota_out.scalar_type() == x.scalar_type() &&
+              iota_out.numel() == x.numel());
+  TORCH_CHECK(x_out.is_contiguous() && iota_out.is_contiguous(), "outputs must be contiguous");
+  if (x_out.numel() == 0) return;
+  x = x.contiguous();
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+  const int es = (int)x.element_size();
+  size_t ws_bytes = yamoe_sort_workspace_bytes((int)x.numel(), es);
+  at::Tensor ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
+  check_rc(yamoe_sort(x.data_ptr(), es, (int)x.numel(), (int)end_bit, x_out.data_ptr(), iota_out.data_ptr(), ws.data_ptr(),
+                      ws_bytes, current_stream()),
+           "yamoe_sort");
+}
+
+void bincount_cumsum_op(at::Tensor input, at::Tensor &output, int64_t minlength) {
+  TORCH_CHECK(input.is_cuda(), "Input must be a GPU tensor");
+  TORCH_CHECK(input.scalar_type() == at::kInt, "Input must be int32");
+  TORCH_CHECK(output.is_cuda() && output.scalar_type() == at::kInt && output.is_contiguous(), "Output must be a contiguous int32 GPU tensor");
+  TORCH_CHECK(output.numel() >= minlength, "Output tensor must have at least minlength elements");
+  input = input.contiguous();
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
+  check_rc(yamoe_bincount_cumsum(input.data_ptr<int>(), (int)input.numel(), output.data_ptr<int>(), (int)output.numel(),
+                                 (int)minlength, current_stream()),
+           "yamoe_bincount_cumsum");
+}
+
+at::Tensor index_select_out_op(at::Tensor out, at::Tensor in, at::Tensor idx_int32) {
+  TORCH_CHECK(in.is_cuda() && idx_int32.is_cuda() && out.is_cuda(), "GPU tensors only");
+  TORCH_CHECK(idx_int32.scalar_type() == at::kInt, "idx must be int32");
+  TORCH_CHECK(in.is_contiguous() && idx_int32.is_contiguous() && out.is_contiguous(), "contiguous required");
+  TORCH_CHECK(out.scalar_type() == in.scalar_type() && out.numel() >= idx_int32.numel(), "out must match input's dtype and idx's length");
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(in.device());
+  check_rc(yamoe_index_select(in.data_ptr(), idx_int32.data_ptr<int>(), out.data_ptr(), idx_int32.numel(),
+                              dtype_code(in, "input"), current_stream()),
+           "yamoe_index_select");
+  return out;
+}
+
+at::Tensor batch_mm_op(at::Tensor x, at::Tensor weights, at::Tensor batch_sizes, at::Tensor output, bool trans_b) {
+  (void)trans_b;  // ignored, as in the reference (csrc/batch_mm.cu:7-31)
+  TORCH_CHECK(x.is_cuda(), "x must be on the GPU");
+  TORCH_CHECK(weights.is_cuda(), "weights must be on the GPU");
+  TORCH_CHECK(batch_sizes.is_cuda(), "batch_sizes must be on the GPU");
+  TORCH_CHECK(x.dim() == 3, "x must be 3D tensor");
+  TORCH_CHECK(weights.dim() == 3, "weights must be 3D tensor");
+  TORCH_CHECK(batch_sizes.dim() == 1, "batch_sizes must be 1D tensor");
+  TORCH_CHECK(x.size(0) == weights.size(0) && x.size(0) == batch_sizes.size(0));
+  TORCH_CHECK(x.size(2) == weights.size(1));
+  const int64_t E = x.size(0), C = x.size(1), Kd = x.size(2), Nd = weights.size(2);
+  TORCH_CHECK(weights.scalar_type() == x.scalar_type() && output.scalar_type() == x.scalar_type(), "dtypes must match");
+  x = x.contiguous();
+  weights = weights.contiguous();
+  if (output.numel() != E * C * Nd) output.resize_({E, C, Nd});
+  TORCH_CHECK(output.is_contiguous(), "output must be contiguous");
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+  size_t ws_bytes = yamoe_batch_mm_workspace_bytes((int)E, (int)C);
+  at::Tensor ws = at::empty({(int64_t)std::max<size_t>(ws_bytes, 1)}, x.options().dtype(at::kByte));
+  check_rc(yamoe_batch_mm(x.data_ptr(), weights.data_ptr(), output.data_ptr(), (int)E, (int)C, (int)Kd, (int)Nd,
+                          dtype_code(x, "x"), ws.data_ptr(), ws_bytes, current_stream()),
+           "yamoe_batch_mm");
+  return output;
+}
+
 }  // namespace
 
 TORCH_LIBRARY(_yamoe_amd_ops, ops) {
+  ops.def("gather(Tensor x, Tensor indices, Tensor bins, Tensor! output, int E, int C, int top_k) -> ()");
+  ops.impl("gather", c10::DispatchKey::CUDA, &gather_op);
+  ops.def("scatter(Tensor src, Tensor indices, Tensor bins, Tensor weights, Tensor! y, int T, int E, int C, "
+          "int top_k) -> ()");
+  ops.impl("scatter", c10::DispatchKey::CUDA, &scatter_op);
+  ops.def("sort(Tensor x, int end_bit, Tensor! x_out, Tensor! iota_out) -> ()");
+  ops.impl("sort", c10::DispatchKey::CUDA, &sort_op);
+  ops.def("bincount_cumsum(Tensor input, Tensor! output, int minlength) -> ()");
+  ops.impl("bincount_cumsum", c10::DispatchKey::CUDA, &bincount_cumsum_op);
+  ops.def("index_select_out(Tensor! out, Tensor input, Tensor idx_int32) -> Tensor");
+  ops.impl("index_select_out", c10::DispatchKey::CUDA, &index_select_out_op);
+  ops.def("batch_mm(Tensor x, Tensor weights, Tensor batch_sizes, Tensor! output, bool trans_b=False) -> Tensor");
+  ops.impl("batch_mm", c10::DispatchKey::CUDA, &batch_mm_op);
+
   ops.def("experts("
           "Tensor hidden_states, "
           "Tensor router_indices, "
