@@ -105,7 +105,8 @@ def test_permute_and_combine(gpu, dtype, T, K, E, H):
                                                (1000, 700, 5, 0), (40, 3, 40, 16)])
 def test_schedule_lists(gpu, N, E, C, stream_rows):
     """The device-built work lists: experts with 1..stream_rows kept rows in the streaming list, the
-    rest cut into 256-row tiles, both in expert order, none dropped, none duplicated."""
+    rest cut into equal row tiles (as few as 256 rows allow, each a multiple of 32 rows but the last), both in
+    expert order, none dropped, none duplicated."""
     from yamoe_amd import _cabi
     rng = np.random.default_rng(N * 7 + E)
     p = rng.random(E) ** 4
@@ -124,8 +125,10 @@ def test_schedule_lists(gpu, N, E, C, stream_rows):
             want_small.append((e, first, kept))
         else:
             g0, n = len(want_tiles), -(-kept // 256)
+            per = min(256, (-(-kept // n) + 31) // 32 * 32)
+            assert (n - 1) * per < kept <= n * per
             for t in range(n):
-                want_tiles.append((e, first + 256 * t, min(256, kept - 256 * t), g0, n))
+                want_tiles.append((e, first + per * t, min(per, kept - per * t), g0, n))
     n_tiles, n_small, n_active, n_kept = sched[:4]
     assert n_tiles == len(want_tiles) and n_small == len(want_small)
     assert n_active == int((np.minimum(r["counts"], C) > 0).sum())

@@ -154,19 +154,25 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const char
   }
 
   u32x4 fa0[NACC], fa1[NACC], fb0[4], fb1[4];
-  // slab s: A pair buffer (s>>1)&1, piece offset 64 bytes (XOR) for the odd slab of the pair
-  auto read_frags = [&](int s, int ks, u32x4 (&fa)[NACC], u32x4 (&fb)[4]) {
-    const char *sb = lds + kBRing + (s & (kBStages - 1)) * kBStageBytes;
-    const char *sa = lds + ((s >> 1) & (kAStages - 1)) * kAStageBytes;
-    const int a_o = a_rd[ks] ^ ((s & 1) << 6);
-#pragma unroll
-    for (int ni = 0; ni < 4; ++ni) {
+  // Operand fragments of one k-step in the order the MFMAs want them: B0, A0, B1, B2, B3, A1, A2, A3.
+  // Slab s sits in A pair buffer (s>>1)&1 (the odd slab of a pair 64 bytes further, by XOR) and B buffer s&3.
+  constexpr int kFrags = NMI > 0 ? 4 + NMI : 0;
+  auto read_frag = [&](int s, int ks, int f, u32x4 (&fa)[NACC], u32x4 (&fb)[4]) {
+    if (f == 1 || f >= 5) {
+      const int mi = f == 1 ? 0 : f - 4;
+      const char *sa = lds + ((s >> 1) & (kAStages - 1)) * kAStageBytes;
+      fa[mi] = *(const u32x4 *)(sa + (a_rd[ks] ^ ((s & 1) << 6)) + mi * 8192);
+    } else {
+      const int ni = f == 0 ? 0 : f - 1;
+      const char *sb = lds + kBRing + (s & (kBStages - 1)) * kBStageBytes;
       u32x2 lo = lds_read_tr16(sb + b_rd[ni] + ks * 8192);
       u32x2 hi = lds_read_tr16(sb + b_rd[ni] + ks * 8192 + 2048);
       fb[ni] = (u32x4){lo[0], lo[1], hi[0], hi[1]};
     }
+  };
+  auto read_frags = [&](int s, int ks, u32x4 (&fa)[NACC], u32x4 (&fb)[4]) {
 #pragma unroll
-    for (int mi = 0; mi < NMI; ++mi) fa[mi] = *(const u32x4 *)(sa + a_o + mi * 8192);
+    for (int f = 0; f < kFrags; ++f) read_frag(s, ks, f, fa, fb);
   };
   auto mma = [&](const u32x4 (&fa)[NACC], const u32x4 (&fb)[4]) {
 #pragma unroll
@@ -174,13 +180,26 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const char
 #pragma unroll
       for (int ni = 0; ni < 4; ++ni) Mma<T>::run(fa[mi], fb[ni], acc[mi][ni]);
   };
+  // copy c of the group issued after the barrier of slab t: (odd t) 8 pieces of A pair (t+1)/2 + 1, then 4
+  // pieces of B slab t + 4
+  auto copy_piece = [&](int t, bool odd, int c) {
+    if (odd && c < 8) {
+      const int pair = (t + 1) / 2 + 1;
+      copy16_to_lds(a_base + (long long)pair * (2 * kBK * (int)sizeof(T)), a_off[c],
+                    lds0 + (uint32_t)(pair & (kAStages - 1)) * kAStageBytes + (uint32_t)(64 * wave + 8 * c) * 128u);
+    } else {
+      const int i = odd ? c - 8 : c, slab = t + kBStages;
+      copy16_to_lds(b_base + (long long)slab * kBK * b_ld_bytes, b_off[i],
+                    lds0 + kBRing + (uint32_t)(slab & (kBStages - 1)) * kBStageBytes + (uint32_t)(8 * wave + 2 * i) * 512u);
+    }
+  };
 
   // ---- pipeline -----------------------------------------------------------------------------------------
   // Copy groups are issued after the mid-slab barrier of slab t: for odd t the A pair (t+1)/2 + 1
   // (8 copies), then B slab t+4 (4 copies).  Copies retire in order and the A pair is needed two slabs
   // later while the B slab has four, so A goes first: a weight fetch that misses to HBM then never
   // delays an activation fetch that hits in L2.  "Slab s+1 has landed" is a bound on how many younger
-  // copies may still be in flight: 8 for odd s, 16 for even s.
+  // copies may still be in flight: 8 for odd s, 16 for even s (4 and 0 once no more copies are issued).
   issue_b(0);
   issue_a(0);
   if (n_slabs > 1) issue_b(1);
@@ -190,33 +209,81 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const char
   __syncthreads();
   read_frags(0, 0, fa0, fb0);
 
-  // One slab: the second k-step's operands are read while the first k-step's MFMAs run; the barrier
-  // sits between the two MFMA groups, followed by the copy issue and the next slab's first reads.
-  auto slab_step = [&](int s, bool odd, bool steady) {
+  // One slab = two k-steps.  The instruction order is fixed by hand, because one wave per SIMD has nobody
+  // to hide behind: every LDS read and every copy is issued in the shadow of an MFMA (an MFMA occupies the
+  // matrix pipe for 8 issue slots), a whole k-step before its result is needed.
+  //   first k-step:  MFMAs on set 0, interleaved with the LDS reads of the second k-step into set 1
+  //   wait for slab s+1's copies; workgroup barrier (after it nobody reads slab s's buffers any more)
+  //   second k-step: MFMAs on set 1, interleaved with this step's copies and the LDS reads of slab s+1
+  //                  (first k-step) into set 0
+  constexpr int kMma = 4 * NMI;
+  constexpr int kSlots = kMma > 2 ? kMma - 2 : 1;  // the last two MFMAs of a k-step carry nothing
+  auto slab_step = [&](int s, auto odd_c, auto issue_c, auto next_c, auto vm_c) {
+    constexpr bool ODD = decltype(odd_c)::value, ISSUE = decltype(issue_c)::value, NEXT = decltype(next_c)::value;
+    constexpr int VM = decltype(vm_c)::value;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
+      if (j < kMma) Mma<T>::run(fa0[j >> 2], fb0[j & 3], acc[j >> 2][j & 3]);
+      if (j < kSlots) {
+#pragma unroll
+        for (int f = j * kFrags / kSlots; f < (j + 1) * kFrags / kSlots; ++f) read_frag(s, 1, f, fa1, fb1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (VM == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else if constexpr (VM == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else if constexpr (VM == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else if constexpr (VM == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    constexpr int kCopies = ISSUE ? (ODD ? 12 : 4) : 0;
+    constexpr int kItems = kCopies + (NEXT ? kFrags : 0);
+#pragma unroll
+    for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
+      if (j < kMma) Mma<T>::run(fa1[j >> 2], fb1[j & 3], acc[j >> 2][j & 3]);
+      if (j < kSlots) {
+#pragma unroll
+        for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
+          if (i < kCopies) copy_piece(s, ODD, i);
+          else read_frag(s + 1, 0, i - kCopies, fa0, fb0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // the same with every decision taken at run time, for contractions shorter than 8 slabs
+  auto slab_step_short = [&](int s, bool odd) {
     read_frags(s, 1, fa1, fb1);
     mma(fa0, fb0);
-    if (steady) {
-      if (odd) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-      else asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-    } else {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
-    // The barrier waits for this wave's LDS reads first, so after it nobody reads slab s's buffers any
-    // more and everybody's share of slab s+1 is visible.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (odd && (steady || s + 3 < n_slabs)) issue_a((s + 1) / 2 + 1);
-    if (steady || s + kBStages < n_slabs) issue_b(s + kBStages);
-    if (steady || s + 1 < n_slabs) read_frags(s + 1, 0, fa0, fb0);
+    if (odd && s + 3 < n_slabs) issue_a((s + 1) / 2 + 1);
+    if (s + kBStages < n_slabs) issue_b(s + kBStages);
+    if (s + 1 < n_slabs) read_frags(s + 1, 0, fa0, fb0);
     mma(fa1, fb1);
   };
-  int s = 0;
-  for (; s + 7 < n_slabs; s += 2) {  // steady state: every copy group exists
-    slab_step(s, false, true);
-    slab_step(s + 1, true, true);
-  }
-  for (; s < n_slabs; s += 2) {
-    slab_step(s, false, false);
-    slab_step(s + 1, true, false);
+  using std::integral_constant;
+  typedef integral_constant<bool, true> yes;
+  typedef integral_constant<bool, false> no;
+  if (n_slabs >= 8) {
+    int s = 0;
+    for (; s + 7 < n_slabs; s += 2) {  // steady state: every copy group exists
+      slab_step(s, no(), yes(), yes(), integral_constant<int, 16>());
+      slab_step(s + 1, yes(), yes(), yes(), integral_constant<int, 8>());
+    }
+    // the last six slabs (s = n_slabs - 6): the last copy group goes out after the barrier of slab n_slabs - 5
+    slab_step(s, no(), yes(), yes(), integral_constant<int, 16>());
+    slab_step(s + 1, yes(), yes(), yes(), integral_constant<int, 8>());
+    slab_step(s + 2, no(), no(), yes(), integral_constant<int, 16>());
+    slab_step(s + 3, yes(), no(), yes(), integral_constant<int, 4>());
+    slab_step(s + 4, no(), no(), yes(), integral_constant<int, 0>());
+    slab_step(s + 5, yes(), no(), no(), integral_constant<int, -1>());
+  } else {
+    for (int s = 0; s < n_slabs; s += 2) {
+      slab_step_short(s, false);
+      slab_step_short(s + 1, true);
+    }
   }
 
   // ---- epilogue -------------------------------------------------------------------------------------

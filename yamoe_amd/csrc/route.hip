@@ -285,9 +285,13 @@ __global__ __launch_bounds__(kWave) void build_schedule_kernel(const int *counts
       s[0] = e; s[1] = first; s[2] = kept; s[3] = 0;
     }
     int gfirst = n_tiles + pos_tiles;
+    // An expert's rows are cut into equal tiles (a multiple of 32 rows, the MFMA block), not into full
+    // tiles plus a remainder: tiles of one expert then advance through the contraction at the same pace
+    // and the weight slabs one of them fetches are still in L2 when the others ask for them.
+    int per_tile = tiles > 0 ? min(kRowTile, (ceil_div(kept, tiles) + 31) & ~31) : 0;
     for (int t = 0; t < tiles; ++t) {
       int *w = row_tiles + 8 * (gfirst + t);
-      w[0] = e; w[1] = first + t * kRowTile; w[2] = min(kRowTile, kept - t * kRowTile); w[3] = gfirst; w[4] = tiles;
+      w[0] = e; w[1] = first + t * per_tile; w[2] = min(per_tile, kept - t * per_tile); w[3] = gfirst; w[4] = tiles;
       w[5] = 0; w[6] = 0; w[7] = 0;
     }
     n_small += tot_small; n_tiles += tot_tiles; n_active += tot_active; n_kept += tot_kept;
