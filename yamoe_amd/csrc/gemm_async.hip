@@ -93,6 +93,12 @@ __device__ inline u32x2 lds_read_tr16(const char *p) {
   return __builtin_bit_cast(u32x2, v);
 }
 
+// what one slab step of the pipeline issues besides its MFMAs
+template <bool P1A_, bool P1B_, bool P2A_, bool P2B_, bool NEXT_, int VM_> struct StepCfg {
+  static constexpr bool P1A = P1A_, P1B = P1B_, P2A = P2A_, P2B = P2B_, NEXT = NEXT_;
+  static constexpr int VM = VM_;
+};
+
 struct TileInfo {
   int expert, row0, rows_valid, n0;
 };
@@ -180,26 +186,25 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const char
 #pragma unroll
       for (int ni = 0; ni < 4; ++ni) Mma<T>::run(fa[mi], fb[ni], acc[mi][ni]);
   };
-  // copy c of the group issued after the barrier of slab t: (odd t) 8 pieces of A pair (t+1)/2 + 1, then 4
-  // pieces of B slab t + 4
-  auto copy_piece = [&](int t, bool odd, int c) {
-    if (odd && c < 8) {
-      const int pair = (t + 1) / 2 + 1;
-      copy16_to_lds(a_base + (long long)pair * (2 * kBK * (int)sizeof(T)), a_off[c],
-                    lds0 + (uint32_t)(pair & (kAStages - 1)) * kAStageBytes + (uint32_t)(64 * wave + 8 * c) * 128u);
-    } else {
-      const int i = odd ? c - 8 : c, slab = t + kBStages;
-      copy16_to_lds(b_base + (long long)slab * kBK * b_ld_bytes, b_off[i],
-                    lds0 + kBRing + (uint32_t)(slab & (kBStages - 1)) * kBStageBytes + (uint32_t)(8 * wave + 2 * i) * 512u);
-    }
+  // One 16-byte-per-lane copy: piece c (0..7) of A pair `pair`, or piece i (0..3) of B slab `slab`.
+  auto copy_a = [&](int pair, int c) {
+    copy16_to_lds(a_base + (long long)pair * (2 * kBK * (int)sizeof(T)), a_off[c],
+                  lds0 + (uint32_t)(pair & (kAStages - 1)) * kAStageBytes + (uint32_t)(64 * wave + 8 * c) * 128u);
+  };
+  auto copy_b = [&](int slab, int i) {
+    copy16_to_lds(b_base + (long long)slab * kBK * b_ld_bytes, b_off[i],
+                  lds0 + kBRing + (uint32_t)(slab & (kBStages - 1)) * kBStageBytes + (uint32_t)(8 * wave + 2 * i) * 512u);
   };
 
   // ---- pipeline -----------------------------------------------------------------------------------------
-  // Copy groups are issued after the mid-slab barrier of slab t: for odd t the A pair (t+1)/2 + 1
-  // (8 copies), then B slab t+4 (4 copies).  Copies retire in order and the A pair is needed two slabs
-  // later while the B slab has four, so A goes first: a weight fetch that misses to HBM then never
-  // delays an activation fetch that hits in L2.  "Slab s+1 has landed" is a bound on how many younger
-  // copies may still be in flight: 8 for odd s, 16 for even s (4 and 0 once no more copies are issued).
+  // A slab is two k-steps with one workgroup barrier between them; after the barrier of slab t nobody reads
+  // slab t's buffers any more.  The L1 path moves 64 bytes per clock into LDS and a slab needs 32 KB of
+  // copies against 1024 clocks of MFMAs, so the copies are spread as evenly as the buffer lifetimes allow:
+  //   second k-step of slab t:  (t odd) first half of A pair (t+1)/2 + 1;  first half of B slab t + 4
+  //   first k-step of slab t:   (t even) second half of A pair t/2 + 1;    second half of B slab t + 3
+  // which is 6, 2, 2, 6 copies per wave over the four k-steps of a slab pair.  Copies retire in order, so
+  // "slab s+1 has landed" is a bound on the number of younger copies in flight at the end of the first
+  // k-step of slab s: 16 for even s, 6 for odd s (2 and 0 for the last two waits).
   issue_b(0);
   issue_a(0);
   if (n_slabs > 1) issue_b(1);
@@ -209,47 +214,54 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const char
   __syncthreads();
   read_frags(0, 0, fa0, fb0);
 
-  // One slab = two k-steps.  The instruction order is fixed by hand, because one wave per SIMD has nobody
-  // to hide behind: every LDS read and every copy is issued in the shadow of an MFMA (an MFMA occupies the
-  // matrix pipe for 8 issue slots), a whole k-step before its result is needed.
-  //   first k-step:  MFMAs on set 0, interleaved with the LDS reads of the second k-step into set 1
-  //   wait for slab s+1's copies; workgroup barrier (after it nobody reads slab s's buffers any more)
-  //   second k-step: MFMAs on set 1, interleaved with this step's copies and the LDS reads of slab s+1
-  //                  (first k-step) into set 0
+  // The instruction order is fixed by hand, because one wave per SIMD has nobody to hide behind: every LDS
+  // read and every copy is issued in the shadow of an MFMA (an MFMA occupies the matrix pipe for 8 issue
+  // slots), a whole k-step before its result is needed.
+  //   first k-step:  MFMAs on set 0 + its copies + the LDS reads of the second k-step into set 1
+  //   wait for slab s+1's copies; workgroup barrier
+  //   second k-step: MFMAs on set 1 + its copies + the LDS reads of slab s+1's first k-step into set 0
   constexpr int kMma = 4 * NMI;
   constexpr int kSlots = kMma > 2 ? kMma - 2 : 1;  // the last two MFMAs of a k-step carry nothing
-  auto slab_step = [&](int s, auto odd_c, auto issue_c, auto next_c, auto vm_c) {
-    constexpr bool ODD = decltype(odd_c)::value, ISSUE = decltype(issue_c)::value, NEXT = decltype(next_c)::value;
-    constexpr int VM = decltype(vm_c)::value;
+  auto slab_step = [&](int s, auto cfg) {
+    typedef decltype(cfg) C;
     __builtin_amdgcn_sched_barrier(0);
+    {
+      constexpr int kA = C::P1A ? 4 : 0, kB = C::P1B ? 2 : 0, kItems = kA + kB + kFrags;
 #pragma unroll
-    for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
-      if (j < kMma) Mma<T>::run(fa0[j >> 2], fb0[j & 3], acc[j >> 2][j & 3]);
-      if (j < kSlots) {
+      for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
+        if (j < kMma) Mma<T>::run(fa0[j >> 2], fb0[j & 3], acc[j >> 2][j & 3]);
+        if (j < kSlots) {
 #pragma unroll
-        for (int f = j * kFrags / kSlots; f < (j + 1) * kFrags / kSlots; ++f) read_frag(s, 1, f, fa1, fb1);
+          for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
+            if (i < kA) copy_a(s / 2 + 1, 4 + i);
+            else if (i < kA + kB) copy_b(s + 3, 2 + i - kA);
+            else read_frag(s, 1, i - kA - kB, fa1, fb1);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
-      __builtin_amdgcn_sched_barrier(0);
     }
-    if constexpr (VM == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-    else if constexpr (VM == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    else if constexpr (VM == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    else if constexpr (VM == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if constexpr (C::VM == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else if constexpr (C::VM == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+    else if constexpr (C::VM == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+    else if constexpr (C::VM == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
-    constexpr int kCopies = ISSUE ? (ODD ? 12 : 4) : 0;
-    constexpr int kItems = kCopies + (NEXT ? kFrags : 0);
+    {
+      constexpr int kA = C::P2A ? 4 : 0, kB = C::P2B ? 2 : 0, kItems = kA + kB + (C::NEXT ? kFrags : 0);
 #pragma unroll
-    for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
-      if (j < kMma) Mma<T>::run(fa1[j >> 2], fb1[j & 3], acc[j >> 2][j & 3]);
-      if (j < kSlots) {
+      for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
+        if (j < kMma) Mma<T>::run(fa1[j >> 2], fb1[j & 3], acc[j >> 2][j & 3]);
+        if (j < kSlots) {
 #pragma unroll
-        for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
-          if (i < kCopies) copy_piece(s, ODD, i);
-          else read_frag(s + 1, 0, i - kCopies, fa0, fb0);
+          for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
+            if (i < kA) copy_a((s + 1) / 2 + 1, i);
+            else if (i < kA + kB) copy_b(s + 4, i - kA);
+            else read_frag(s + 1, 0, i - kA - kB, fa0, fb0);
+          }
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
-      __builtin_amdgcn_sched_barrier(0);
     }
   };
   // the same with every decision taken at run time, for contractions shorter than 8 slabs
@@ -263,22 +275,22 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const char
     if (s + 1 < n_slabs) read_frags(s + 1, 0, fa0, fb0);
     mma(fa1, fb1);
   };
-  using std::integral_constant;
-  typedef integral_constant<bool, true> yes;
-  typedef integral_constant<bool, false> no;
   if (n_slabs >= 8) {
-    int s = 0;
-    for (; s + 7 < n_slabs; s += 2) {  // steady state: every copy group exists
-      slab_step(s, no(), yes(), yes(), integral_constant<int, 16>());
-      slab_step(s + 1, yes(), yes(), yes(), integral_constant<int, 8>());
+    // copies of the (first, second) k-step: A half, B half; whether slab s+1 is read; the vmcnt bound (-1: no wait)
+    slab_step(0, StepCfg<false, false, false, true, true, -1>());
+    slab_step(1, StepCfg<false, true, true, true, true, -1>());
+    int s = 2;
+    for (; s + 7 < n_slabs; s += 2) {  // steady state
+      slab_step(s, StepCfg<true, true, false, true, true, 16>());
+      slab_step(s + 1, StepCfg<false, true, true, true, true, 6>());
     }
-    // the last six slabs (s = n_slabs - 6): the last copy group goes out after the barrier of slab n_slabs - 5
-    slab_step(s, no(), yes(), yes(), integral_constant<int, 16>());
-    slab_step(s + 1, yes(), yes(), yes(), integral_constant<int, 8>());
-    slab_step(s + 2, no(), no(), yes(), integral_constant<int, 16>());
-    slab_step(s + 3, yes(), no(), yes(), integral_constant<int, 4>());
-    slab_step(s + 4, no(), no(), yes(), integral_constant<int, 0>());
-    slab_step(s + 5, yes(), no(), no(), integral_constant<int, -1>());
+    // the last six slabs (s = n_slabs - 6): the last copies go out in the first k-step of slab n_slabs - 4
+    slab_step(s, StepCfg<true, true, false, true, true, 16>());
+    slab_step(s + 1, StepCfg<false, true, true, true, true, 6>());
+    slab_step(s + 2, StepCfg<true, true, false, false, true, 16>());
+    slab_step(s + 3, StepCfg<false, false, false, false, true, 2>());
+    slab_step(s + 4, StepCfg<false, false, false, false, true, 0>());
+    slab_step(s + 5, StepCfg<false, false, false, false, false, -1>());
   } else {
     for (int s = 0; s < n_slabs; s += 2) {
       slab_step_short(s, false);
