@@ -62,6 +62,24 @@ def test_forward_capacity_drop_and_slot_weights(gpu, dtype):
     assert torch.equal(run_op(d2, 60, gpu), base)
 
 
+def test_forward_uneven_tile_costs(gpu):
+    """Eight experts with 2048 rows each and 56 experts with 20 rows each: the shares of the tile list that the
+    8 XCDs get are equal in cost, so the shares made of small tiles hold more tiles than the grid has workgroups
+    per XCD and the excess goes to workgroups of other XCDs."""
+    E, H, I = 64, 128, 128
+    ids = np.concatenate([np.repeat(np.arange(8), 2048), np.repeat(np.arange(8, 64), 20)])
+    rng = np.random.default_rng(3)
+    rng.shuffle(ids)
+    T = len(ids)
+    d = make_inputs(T, H, I, E, 1, torch.bfloat16, seed=5, w_std=0.05, bias_std=0.1)
+    d["router_indices"] = torch.from_numpy(ids.astype(np.int64)).reshape(T, 1)
+    d["routing_weights"] = torch.rand(T, E, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+    got = run_op(d, T, gpu)
+    want = oracle_forward(d, T)
+    tol = REL_L2_TOL[torch.bfloat16]
+    assert report("uneven tile costs", got.double(), want.double(), tol) < tol
+
+
 def test_forward_special_cases(gpu):
     """Structure checks that do not depend on the oracle's matmul: one-hot routing returns the
     expert's row, zero weights reduce to the bias closed form, an unused expert changes nothing."""

@@ -134,7 +134,34 @@ def test_schedule_lists(gpu, N, E, C, stream_rows):
     assert n_active == int((np.minimum(r["counts"], C) > 0).sum())
     assert n_kept == int(np.minimum(r["counts"], C).sum())
     max_tiles = N // 256 + min(N, E) + 1
-    tiles = sched[8:8 + 8 * n_tiles].reshape(-1, 8)[:, :5]
+    tiles = sched[48:48 + 8 * n_tiles].reshape(-1, 8)[:, :5]
     assert [tuple(t) for t in tiles.tolist()] == want_tiles
-    small = sched[8 + 8 * max_tiles:8 + 8 * max_tiles + 4 * n_small].reshape(-1, 4)[:, :3]
+    small = sched[48 + 8 * max_tiles:48 + 8 * max_tiles + 4 * n_small].reshape(-1, 4)[:, :3]
     assert [tuple(t) for t in small.tolist()] == want_small
+    # The cut table: 9 cuts that split the tile list into 8 shares of (nearly) equal cost for any number of
+    # column tiles; every cut lies on an (expert, column tile) boundary and the cuts are monotone.
+    weight = lambda rows: 3 + 2 * ((rows + 63) // 64)
+    w_tiles = [weight(t[2]) for t in want_tiles]
+    assert sched[4] == sum(w_tiles)
+    for n_col in (1, 12, 23):
+        cuts = []
+        for x in range(9):
+            first, frac, _, cnt = sched[8 + 4 * x:12 + 4 * x].tolist()
+            assert 0 <= frac < 65536
+            cuts.append(first * n_col + ((frac * n_col) >> 16) * cnt)
+        assert cuts[0] == 0 and cuts[8] == len(want_tiles) * n_col
+        assert all(a <= b for a, b in zip(cuts, cuts[1:]))
+        # flat list: group-major, then column tile, then the group's row tiles
+        flat, bounds = [], {0}
+        g = 0
+        while g < len(want_tiles):
+            cnt = want_tiles[g][4]
+            for c in range(n_col):
+                flat += w_tiles[g:g + cnt]
+                bounds.add(len(flat))
+            g += cnt
+        assert all(c in bounds for c in cuts)
+        if flat:
+            shares = [sum(flat[a:b]) for a, b in zip(cuts, cuts[1:])]
+            biggest_unit = max(sum(w_tiles[g:g + want_tiles[g][4]]) for g in range(len(want_tiles)))
+            assert max(shares) - sum(flat) / 8 <= 2 * biggest_unit + 1e-9

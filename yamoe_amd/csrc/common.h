@@ -78,11 +78,28 @@ __device__ inline void glu_backward(float G, float U, float dh, float &dG, float
 //   [1] n_small       number of experts on the weight-streaming path
 //   [2] n_active      experts with at least one kept row
 //   [3] n_kept        total kept rows
-//   [8 ...)           row tiles: 8 words each  {expert, first sorted row, valid rows,
+//   [4] weight_total  sum of the row-tile cost weights (sched_tile_weight)
+//   [8 + 4x ...)      x = 0..8: where the tile list is cut so that each of the 8 XCDs gets the same share of
+//                     the cost: {first row tile of the expert the cut falls in, f, 0, row tiles of that
+//                     expert}, f = the cut's position inside that expert's tiles in 1/65536ths; in a GEMM
+//                     with n column tiles the cut is at flat tile index
+//                     first * n + ((f * n) >> 16) * row_tiles, i.e. on a column-tile boundary of that expert
+//   [48 ...)          row tiles: 8 words each  {expert, first sorted row, valid rows,
 //                       index of the expert's first row tile, number of row tiles of the expert, 0,0,0}
 //   then              small experts: 4 words each {expert, first sorted row, valid rows, 0}
 constexpr int kRowTile = 256;  // rows of one MFMA row tile
-constexpr int kSchedHeader = 8;
+constexpr int kSchedHeader = 48;
+constexpr int kSchedCuts = 8;  // word offset of the XCD cut table
+constexpr int kXcds = 8;
+
+// Relative cost of one row tile in the MFMA kernels: a fixed part (prologue, epilogue, copies of the weight
+// slabs) plus one part per 64 rows (the MFMA blocks of the slower wave row).
+__host__ __device__ inline int sched_tile_weight(int rows) { return 3 + 2 * ((rows + 63) / 64); }
+// flat tile index of cut x of the schedule for a GEMM with n_col_tiles column tiles
+__host__ __device__ inline int sched_cut(const int *sched, int x, int n_col_tiles) {
+  const int *c = sched + kSchedCuts + 4 * x;
+  return c[0] * n_col_tiles + ((c[1] * n_col_tiles) >> 16) * c[3];
+}
 
 __host__ __device__ inline int sched_max_row_tiles(int N, int E) {
   // every expert with kept rows adds at most one partly filled tile

@@ -38,7 +38,6 @@ constexpr int kGemmThreads = 256;
 constexpr int kRowBytes = 128;                 // bytes of one LDS tile row (one K slab)
 constexpr int kTileBytes = kBM * kRowBytes;    // 32 KB per operand per stage
 constexpr int kGemmLds = 4 * kTileBytes;       // A,B x 2 stages = 128 KB
-constexpr int kXcds = 8;
 
 static_assert(kBM == kRowTile, "row tiles of the schedule must match the GEMM tile");
 

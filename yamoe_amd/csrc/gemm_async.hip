@@ -45,7 +45,6 @@ constexpr int kBRing = kAStages * kAStageBytes;    // byte offset of the B ring
 constexpr int kRingBytes = kBRing + kBStages * kBStageBytes;  // 128 KB
 constexpr int kStagingBytes = kBM * (kBN * 2 + 16);            // output tile staged for the row-wise store
 constexpr int kLds = kStagingBytes > kRingBytes ? kStagingBytes : kRingBytes;
-constexpr int kXcds = 8;
 
 static_assert(kBM == kRowTile, "row tiles of the schedule must match the GEMM tile");
 
@@ -104,9 +103,10 @@ struct TileInfo {
 };
 
 template <typename T, int EPI, int NMI>
-__device__ inline void run_tile(const Args &args, const TileInfo &ti, const char *a_base, const uint32_t (&a_off)[8],
-                                const char *b_base, const uint32_t (&b_off)[4], long long b_ld_bytes) {
-  const int tid = threadIdx.x, lane = tid & 63;
+__device__ inline void run_tile(const Args &args, const TileInfo &ti, const int tid, const char *a_base,
+                                const uint32_t (&a_off)[8], const char *b_base, const uint32_t (&b_off)[4],
+                                long long b_ld_bytes) {
+  const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in a scalar register
   const int wm = wave >> 1, wn = wave & 1;
   constexpr int NACC = NMI > 0 ? NMI : 1;
@@ -321,6 +321,9 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const char
   // natural column order: value = acc + bias[column]   (the plain product, or the pre-activations)
   auto stage_biased = [&]() {
     constexpr int stride = kBN * 2 + 16;
+    // one address per lane; everything else is a compile-time offset (two bases: the offset field holds 16 bits)
+    char *lp0 = lds + (wm * 32 + rsub) * stride + (wn * 128 + rl) * 2;
+    char *lp1 = lp0 + 128 * stride;
 #pragma unroll
     for (int ni = 0; ni < 4; ++ni) {
       int lc = wn * 128 + ni * 32 + rl;
@@ -331,8 +334,8 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const char
       for (int mi = 0; mi < NMI; ++mi)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          int r = (mi * 2 + wm) * 32 + 8 * (v >> 2) + rsub + (v & 3);
-          *(T *)(lds + r * stride + lc * 2) = ElemTraits<T>::from_f32(acc[mi][ni][v] + bias);
+          char *q = (mi < 2 ? lp0 : lp1) + ((mi & 1) * 64 + 8 * (v >> 2) + (v & 3)) * stride + ni * 64;
+          *(T *)q = ElemTraits<T>::from_f32(acc[mi][ni][v] + bias);
         }
     }
   };
@@ -353,6 +356,8 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const char
     // rows (v, v+1) the even lane finishes row v and the odd lane row v+1 after one DPP swap.
     constexpr int stride = (kBN / 2) * 2 + 16;
     const bool odd = lane & 1;
+    // tile row (mi*2+wm)*32 + 8*(v/4) + rsub + v%4 with v = 2u + odd; activation column (wn*128 + ni*32 + rl) / 2
+    char *lp = lds + (wm * 32 + rsub + (odd ? 1 : 0)) * stride + wn * 128 + (rl & ~1);
 #pragma unroll
     for (int ni = 0; ni < 4; ++ni) {
       int lc = wn * 128 + ni * 32 + (rl & ~1);  // tile column of the gate of this lane's pair
@@ -371,9 +376,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const char
           float recv = __builtin_bit_cast(
               float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, send), 0xB1 /* quad_perm [1,0,3,2] */, 0xF, 0xF, true));
           float G = (odd ? recv : xe) + bg, U = (odd ? xo : recv) + bu;
-          int v = 2 * u + (odd ? 1 : 0);
-          int r = (mi * 2 + wm) * 32 + 8 * (v >> 2) + rsub + (v & 3);
-          *(T *)(lds + r * stride + (lc >> 1) * 2) = ElemTraits<T>::from_f32(glu_forward(G, U));
+          *(T *)(lp + (mi * 64 + 8 * (u >> 1) + 2 * (u & 1)) * stride + ni * 32) = ElemTraits<T>::from_f32(glu_forward(G, U));
         }
       }
     }
@@ -384,18 +387,41 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const char
 
 template <typename T, int EPI, bool GATHER>
 __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1;
 
+  // Workgroup b runs on XCD b % 8 and takes tile b / 8 of that XCD's share of the tile list.  The shares have
+  // equal cost, not equal length, and are cut on (expert, column tile) boundaries, so the row tiles that read
+  // the same weight slabs meet in one L2.  A share longer than gridDim.x / 8 hands its excess to the workgroups
+  // of shorter shares (the grid has at least as many workgroups as there are tiles).
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1;
+  int L;
+  {
+    const int xcd = blockIdx.x % kXcds, i = blockIdx.x / kXcds, slots = gridDim.x / kXcds;
+    const int first = sched_cut(args.sched, xcd, args.n_col_tiles);
+    const int count = sched_cut(args.sched, xcd + 1, args.n_col_tiles) - first;
+    if (i < count) {
+      L = first + i;
+    } else {
+      int cut[kXcds + 1];
+#pragma unroll
+      for (int x = 0; x <= kXcds; ++x) cut[x] = sched_cut(args.sched, x, args.n_col_tiles);
+      int rank = i - count;  // rank of this workgroup among the idle ones
+#pragma unroll
+      for (int x = 0; x < kXcds; ++x)
+        if (x < xcd) rank += max(slots - (cut[x + 1] - cut[x]), 0);
+      L = -1;
+#pragma unroll
+      for (int x = 0; x < kXcds; ++x) {
+        int excess = max(cut[x + 1] - cut[x] - slots, 0);
+        if (L < 0) {
+          if (rank < excess) L = cut[x] + slots + rank;
+          else rank -= excess;
+        }
+      }
+      if (L < 0) return;
+    }
+  }
   TileInfo ti;
   {
-    int n_row_tiles = args.sched[0];
-    int total = n_row_tiles * args.n_col_tiles;
-    int total8 = (total + kXcds - 1) / kXcds * kXcds;
-    int b = blockIdx.x;
-    if (b >= total8) return;
-    int L = (b % kXcds) * (total8 / kXcds) + b / kXcds;
-    if (L >= total) return;
     const int *tiles = args.sched + kSchedHeader;
     int t0 = L / args.n_col_tiles;
     int gfirst = tiles[8 * t0 + 3], gcount = tiles[8 * t0 + 4];
@@ -435,11 +461,11 @@ __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
   const int n_blocks32 = (ti.rows_valid + 31) >> 5;
   const int n_mi = (n_blocks32 - wm + 1) >> 1;
   switch (n_mi) {
-    case 4: run_tile<T, EPI, 4>(args, ti, a_base, a_off, b_base, b_off, b_ld_bytes); break;
-    case 3: run_tile<T, EPI, 3>(args, ti, a_base, a_off, b_base, b_off, b_ld_bytes); break;
-    case 2: run_tile<T, EPI, 2>(args, ti, a_base, a_off, b_base, b_off, b_ld_bytes); break;
-    case 1: run_tile<T, EPI, 1>(args, ti, a_base, a_off, b_base, b_off, b_ld_bytes); break;
-    default: run_tile<T, EPI, 0>(args, ti, a_base, a_off, b_base, b_off, b_ld_bytes); break;
+    case 4: run_tile<T, EPI, 4>(args, ti, tid, a_base, a_off, b_base, b_off, b_ld_bytes); break;
+    case 3: run_tile<T, EPI, 3>(args, ti, tid, a_base, a_off, b_base, b_off, b_ld_bytes); break;
+    case 2: run_tile<T, EPI, 2>(args, ti, tid, a_base, a_off, b_base, b_off, b_ld_bytes); break;
+    case 1: run_tile<T, EPI, 1>(args, ti, tid, a_base, a_off, b_base, b_off, b_ld_bytes); break;
+    default: run_tile<T, EPI, 0>(args, ti, tid, a_base, a_off, b_base, b_off, b_ld_bytes); break;
   }
 }
 

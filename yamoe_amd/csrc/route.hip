@@ -296,9 +296,43 @@ __global__ __launch_bounds__(kWave) void build_schedule_kernel(const int *counts
     }
     n_small += tot_small; n_tiles += tot_tiles; n_active += tot_active; n_kept += tot_kept;
   }
+  // Second pass: cut the tile list into 8 shares of equal cost.  Groups (experts with row tiles) are weighed
+  // by the sum of their tiles' weights; cut x falls into the group that contains x/8 of the total.
+  int w_total = 0;
+  for (int pass = 0; pass < 2; ++pass) {
+    int w_before = 0, t_before = 0;
+    for (int base = 0; base < E; base += kWave) {
+      int e = base + lane;
+      int kept = e < E ? min(counts[e], capacity) : 0;
+      if (kept < 0) kept = 0;
+      int is_small = kept > 0 && kept <= stream_max_rows;
+      int tiles = (kept > 0 && !is_small) ? ceil_div(kept, kRowTile) : 0;
+      int per_tile = tiles > 0 ? min(kRowTile, (ceil_div(kept, tiles) + 31) & ~31) : 0;
+      int w = tiles > 0 ? (tiles - 1) * sched_tile_weight(per_tile) + sched_tile_weight(kept - (tiles - 1) * per_tile) : 0;
+      int tot_w, tot_t;
+      int w_pre = w_before + wave_exclusive_scan(w, lane, tot_w);
+      int t_pre = t_before + wave_exclusive_scan(tiles, lane, tot_t);
+      if (pass == 1 && tiles > 0) {
+        for (int x = 0; x < kXcds; ++x) {
+          long long t = (long long)x * w_total;  // compare x * W / 8 with the group's weight interval, times 8
+          if (t >= 8ll * w_pre && t < 8ll * (w_pre + w)) {
+            int *c = sched + kSchedCuts + 4 * x;
+            c[0] = t_pre; c[1] = (int)(((t - 8ll * w_pre) << 16) / (8ll * w)); c[2] = 0; c[3] = tiles;
+          }
+        }
+      }
+      w_before += tot_w; t_before += tot_t;
+    }
+    if (pass == 0) w_total = w_before;
+  }
   if (lane == 0) {
     sched[0] = n_tiles; sched[1] = n_small; sched[2] = n_active; sched[3] = n_kept;
-    sched[4] = 0; sched[5] = 0; sched[6] = 0; sched[7] = 0;
+    sched[4] = w_total; sched[5] = 0; sched[6] = 0; sched[7] = 0;
+    int *c = sched + kSchedCuts + 4 * kXcds;  // the end of the list
+    c[0] = n_tiles; c[1] = 0; c[2] = 0; c[3] = 0;
+    if (w_total == 0)
+      for (int x = 0; x < kXcds; ++x) { int *cx = sched + kSchedCuts + 4 * x; cx[0] = 0; cx[1] = 0; cx[2] = 0; cx[3] = 0; }
+    for (int i = kSchedCuts + 4 * (kXcds + 1); i < kSchedHeader; ++i) sched[i] = 0;
   }
 }
 
