@@ -57,6 +57,8 @@ int gemm_async_gate_up(const void *, const int *, const void *, const void *, vo
                        int, int, int, hipStream_t);
 template <typename T>
 int gemm_async_down(const void *, const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);
+template <typename T>
+int gemm_async_dgrad(const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);
 bool gemm_async_supported(int Kd, int Nd, int lda, int ldb, long long a_span_bytes);
 
 template <typename T> struct HasStreamPath { static constexpr bool value = sizeof(T) == 2; };
@@ -80,6 +82,15 @@ static int tiles_down(const void *act, const void *w, const void *bias, void *y,
     if (gemm_async_supported(I, H, I, H, 0)) return gemm_async_down<T>(act, w, bias, y, sched, N, E, H, I, stream);
   }
   return gemm_down<T>(act, w, bias, y, sched, N, E, H, I, stream);
+}
+
+template <typename T>
+static int tiles_dgrad(const void *g, const void *w, void *out, const void *sched, int N, int E, int Kd, int Nd,
+                       hipStream_t stream) {
+  if constexpr (sizeof(T) == 2) {
+    if (gemm_async_supported(Kd, Nd, Kd, Kd, 0)) return gemm_async_dgrad<T>(g, w, out, sched, N, E, Kd, Nd, stream);
+  }
+  return gemm_dgrad<T>(g, w, out, sched, N, E, Kd, Nd, stream);
 }
 
 __global__ void fill_zero_kernel(uint32_t *p, long long n_words) {
@@ -237,13 +248,13 @@ static int backward_impl(const yamoe_problem *p, const void *gy, const void *x, 
                                        b.g_y_perm, d_rw, N, p->K, E, H, stream));
   // down projection
   YAMOE_TRY(launch_expert_colsum<T>(b.g_y_perm, b.f.counts, b.f.offsets, cap, d_bd, E, H, stream));
-  YAMOE_TRY(gemm_dgrad<T>(b.g_y_perm, wd, b.d_act, b.f.schedule, N, E, /*Kd=*/H, /*Nd=*/I, stream));
+  YAMOE_TRY(tiles_dgrad<T>(b.g_y_perm, wd, b.d_act, b.f.schedule, N, E, /*Kd=*/H, /*Nd=*/I, stream));
   YAMOE_TRY(gemm_wgrad<T>(b.f.act, b.g_y_perm, d_wd, b.f.counts, b.f.offsets, cap, E, /*Md=*/I, /*Nd=*/H, stream));
   // GLU
   YAMOE_TRY(glu_backward_rows<T>(b.d_act, b.pre, b.d_pre, (long long)N * I, stream));
   // gate_up projection
   YAMOE_TRY(launch_expert_colsum<T>(b.d_pre, b.f.counts, b.f.offsets, cap, d_bgu, E, 2 * I, stream));
-  YAMOE_TRY(gemm_dgrad<T>(b.d_pre, wgu, b.d_x_perm, b.f.schedule, N, E, /*Kd=*/2 * I, /*Nd=*/H, stream));
+  YAMOE_TRY(tiles_dgrad<T>(b.d_pre, wgu, b.d_x_perm, b.f.schedule, N, E, /*Kd=*/2 * I, /*Nd=*/H, stream));
   YAMOE_TRY(gemm_wgrad<T>(b.x_perm, b.d_pre, d_wgu, b.f.counts, b.f.offsets, cap, E, /*Md=*/H, /*Nd=*/2 * I, stream));
   // permute backward: d_hidden[t] = sum_k d_x_perm[inv_pos[t,k]]
   YAMOE_TRY(launch_combine<T>(b.d_x_perm, b.f.inv_pos, idx, p->idx_i64, nullptr, p->K, d_x, p->T, p->K, E, H, stream));

@@ -102,10 +102,10 @@ struct TileInfo {
   int expert, row0, rows_valid, n0;
 };
 
-template <typename T, int EPI, int NMI>
+template <typename T, int EPI, int NMI, bool BNK>
 __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int tid, const char *a_base,
                                 const uint32_t (&a_off)[8], const char *b_base, const uint32_t (&b_off)[4],
-                                long long b_ld_bytes) {
+                                long long b_slab_bytes) {
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in a scalar register
   const int wm = wave >> 1, wn = wave & 1;
@@ -135,7 +135,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
   // B slab: this wave fills k rows 8*wave + 2*i + (lane >> 5), 512 bytes each.
   auto issue_b = [&](int slab) {
     const uint32_t stage = lds0 + kBRing + (uint32_t)(slab & (kBStages - 1)) * kBStageBytes;
-    const char *bb = b_base + (long long)slab * kBK * b_ld_bytes;
+    const char *bb = b_base + (long long)slab * b_slab_bytes;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       copy16_to_lds(bb, b_off[i], stage + (uint32_t)(8 * wave + 2 * i) * 512u);
@@ -158,6 +158,11 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
     int piece = (col >> 3) ^ (j4 << 2);
     b_rd[ni] = (g * 8 + j4) * 512 + (piece << 4) + (col & 7) * 2;
   }
+  // B operand of a [n][k] tile (BNK): 64-byte rows, row wn*128 + ni*32 + lane%32, piece ks*2 + lane/32 at
+  // position piece ^ ((row >> 2) & 3); one 16-byte read per operand, like A.
+  int b_rdk[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) b_rdk[ks] = (wn * 128 + rl) * 64 + (((ks * 2 + g) ^ ((rl >> 2) & 3)) << 4);
 
   u32x4 fa0[NACC], fa1[NACC], fb0[4], fb1[4];
   // Operand fragments of one k-step in the order the MFMAs want them: B0, A0, B1, B2, B3, A1, A2, A3.
@@ -171,9 +176,13 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
     } else {
       const int ni = f == 0 ? 0 : f - 1;
       const char *sb = lds + kBRing + (s & (kBStages - 1)) * kBStageBytes;
-      u32x2 lo = lds_read_tr16(sb + b_rd[ni] + ks * 8192);
-      u32x2 hi = lds_read_tr16(sb + b_rd[ni] + ks * 8192 + 2048);
-      fb[ni] = (u32x4){lo[0], lo[1], hi[0], hi[1]};
+      if constexpr (BNK) {
+        fb[ni] = *(const u32x4 *)(sb + b_rdk[ks] + ni * 2048);
+      } else {
+        u32x2 lo = lds_read_tr16(sb + b_rd[ni] + ks * 8192);
+        u32x2 hi = lds_read_tr16(sb + b_rd[ni] + ks * 8192 + 2048);
+        fb[ni] = (u32x4){lo[0], lo[1], hi[0], hi[1]};
+      }
     }
   };
   auto read_frags = [&](int s, int ks, u32x4 (&fa)[NACC], u32x4 (&fb)[4]) {
@@ -192,7 +201,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
                   lds0 + (uint32_t)(pair & (kAStages - 1)) * kAStageBytes + (uint32_t)(64 * wave + 8 * c) * 128u);
   };
   auto copy_b = [&](int slab, int i) {
-    copy16_to_lds(b_base + (long long)slab * kBK * b_ld_bytes, b_off[i],
+    copy16_to_lds(b_base + (long long)slab * b_slab_bytes, b_off[i],
                   lds0 + kBRing + (uint32_t)(slab & (kBStages - 1)) * kBStageBytes + (uint32_t)(8 * wave + 2 * i) * 512u);
   };
 
@@ -385,7 +394,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
   }
 }
 
-template <typename T, int EPI, bool GATHER>
+template <typename T, int EPI, bool GATHER, bool BNK>
 __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
 
   // Workgroup b runs on XCD b % 8 and takes tile b / 8 of that XCD's share of the tile list.  The shares have
@@ -445,33 +454,50 @@ __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
   }
   const char *a_base = (const char *)((const T *)args.A + (GATHER ? 0ll : (long long)ti.row0 * args.lda));
 
-  // B copies: k rows 8*wave + 2*i + (lane >> 5); LDS position lane & 31 holds piece pos ^ ((k & 3) << 2)
   const long long b_ld_bytes = (long long)args.ldb * (long long)sizeof(T);
   uint32_t b_off[4];
+  const char *b_base;
+  long long b_slab_bytes;
+  if constexpr (BNK) {
+    // B is [n][k] (k-contiguous rows, one per output column): rows 64*wave + 16*i + (lane >> 2), 64 bytes of each
+    // per slab; LDS position lane & 3 holds piece pos ^ ((row >> 2) & 3)
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    int k = 8 * wave + 2 * i + (lane >> 5);
-    int piece = (lane & 31) ^ ((k & 3) << 2);
-    int col = ti.n0 + piece * 8;
-    if (col >= args.Nd) col = ti.n0;  // columns past the end re-read valid ones; never stored
-    b_off[i] = (uint32_t)(k * b_ld_bytes + (long long)(col - ti.n0) * (long long)sizeof(T));
+    for (int i = 0; i < 4; ++i) {
+      int row = 64 * wave + 16 * i + (lane >> 2);
+      int piece = (lane & 3) ^ ((row >> 2) & 3);
+      int r = min(row, args.Nd - 1 - ti.n0);  // columns past the end re-read the last one; never stored
+      b_off[i] = (uint32_t)(r * b_ld_bytes + piece * 16);
+    }
+    b_base = (const char *)((const T *)args.B + (long long)ti.expert * args.b_expert_stride + (long long)ti.n0 * args.ldb);
+    b_slab_bytes = kBK * (long long)sizeof(T);
+  } else {
+    // B is [k][n]: k rows 8*wave + 2*i + (lane >> 5); LDS position lane & 31 holds piece pos ^ ((k & 3) << 2)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int k = 8 * wave + 2 * i + (lane >> 5);
+      int piece = (lane & 31) ^ ((k & 3) << 2);
+      int col = ti.n0 + piece * 8;
+      if (col >= args.Nd) col = ti.n0;  // columns past the end re-read valid ones; never stored
+      b_off[i] = (uint32_t)(k * b_ld_bytes + (long long)(col - ti.n0) * (long long)sizeof(T));
+    }
+    b_base = (const char *)((const T *)args.B + (long long)ti.expert * args.b_expert_stride + ti.n0);
+    b_slab_bytes = kBK * b_ld_bytes;
   }
-  const char *b_base = (const char *)((const T *)args.B + (long long)ti.expert * args.b_expert_stride + ti.n0);
 
   const int n_blocks32 = (ti.rows_valid + 31) >> 5;
   const int n_mi = (n_blocks32 - wm + 1) >> 1;
   switch (n_mi) {
-    case 4: run_tile<T, EPI, 4>(args, ti, tid, a_base, a_off, b_base, b_off, b_ld_bytes); break;
-    case 3: run_tile<T, EPI, 3>(args, ti, tid, a_base, a_off, b_base, b_off, b_ld_bytes); break;
-    case 2: run_tile<T, EPI, 2>(args, ti, tid, a_base, a_off, b_base, b_off, b_ld_bytes); break;
-    case 1: run_tile<T, EPI, 1>(args, ti, tid, a_base, a_off, b_base, b_off, b_ld_bytes); break;
-    default: run_tile<T, EPI, 0>(args, ti, tid, a_base, a_off, b_base, b_off, b_ld_bytes); break;
+    case 4: run_tile<T, EPI, 4, BNK>(args, ti, tid, a_base, a_off, b_base, b_off, b_slab_bytes); break;
+    case 3: run_tile<T, EPI, 3, BNK>(args, ti, tid, a_base, a_off, b_base, b_off, b_slab_bytes); break;
+    case 2: run_tile<T, EPI, 2, BNK>(args, ti, tid, a_base, a_off, b_base, b_off, b_slab_bytes); break;
+    case 1: run_tile<T, EPI, 1, BNK>(args, ti, tid, a_base, a_off, b_base, b_off, b_slab_bytes); break;
+    default: run_tile<T, EPI, 0, BNK>(args, ti, tid, a_base, a_off, b_base, b_off, b_slab_bytes); break;
   }
 }
 
-template <typename T, int EPI, bool GATHER>
+template <typename T, int EPI, bool GATHER, bool BNK>
 static int launch(const Args &args, int max_row_tiles, hipStream_t stream) {
-  auto kernel = gemm_async_kernel<T, EPI, GATHER>;
+  auto kernel = gemm_async_kernel<T, EPI, GATHER, BNK>;
   static bool attr_done = false;  // benign race: the attribute call is idempotent
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
@@ -505,7 +531,7 @@ int gemm_async_gate_up(const void *x, const int *sorted_idx, const void *w, cons
   a.Kd = H; a.Nd = 2 * I; a.lda = H; a.ldb = 2 * I; a.ldc = I;
   a.b_expert_stride = (long long)H * 2 * I;
   a.n_col_tiles = ceil_div(2 * I, async::kBN);
-  return async::launch<T, async::EPI_GLU, true>(a, sched_max_row_tiles(N, E), stream);
+  return async::launch<T, async::EPI_GLU, true, false>(a, sched_max_row_tiles(N, E), stream);
 }
 
 template <typename T>
@@ -516,14 +542,28 @@ int gemm_async_down(const void *act, const void *w, const void *bias, void *y, c
   a.Kd = I; a.Nd = H; a.lda = I; a.ldb = H; a.ldc = H;
   a.b_expert_stride = (long long)I * H;
   a.n_col_tiles = ceil_div(H, async::kBN);
-  return async::launch<T, async::EPI_STORE, false>(a, sched_max_row_tiles(N, E), stream);
+  return async::launch<T, async::EPI_STORE, false, false>(a, sched_max_row_tiles(N, E), stream);
+}
+
+// C[rows, Nd] = A[rows, Kd] * W[e]^T with W[e] stored [Nd, Kd]: the input gradients of both projections
+// (csrc/experts_backward.cu:279-282, 309-311), without materialising a transposed weight.
+template <typename T>
+int gemm_async_dgrad(const void *g, const void *w, void *out, const void *sched, int N, int E, int Kd, int Nd,
+                     hipStream_t stream) {
+  async::Args a = {};
+  a.A = g; a.B = w; a.bias = nullptr; a.C = out; a.sched = (const int *)sched;
+  a.Kd = Kd; a.Nd = Nd; a.lda = Kd; a.ldb = Kd; a.ldc = Nd;
+  a.b_expert_stride = (long long)Nd * Kd;
+  a.n_col_tiles = ceil_div(Nd, async::kBN);
+  return async::launch<T, async::EPI_STORE, false, true>(a, sched_max_row_tiles(N, E), stream);
 }
 
 #define YAMOE_INSTANTIATE_ASYNC(T)                                                                               \
   template int gemm_async_gate_up<T>(const void *, const int *, const void *, const void *, void *, void *,      \
                                      const void *, int, int, int, int, int, hipStream_t);                        \
   template int gemm_async_down<T>(const void *, const void *, const void *, void *, const void *, int, int, int, \
-                                  int, hipStream_t);
+                                  int, hipStream_t);                                                             \
+  template int gemm_async_dgrad<T>(const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);
 YAMOE_INSTANTIATE_ASYNC(bf16_t)
 YAMOE_INSTANTIATE_ASYNC(f16_t)
 

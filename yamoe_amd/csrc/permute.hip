@@ -150,13 +150,61 @@ __global__ __launch_bounds__(kRowThreads) void combine_backward_kernel(
 
 // Column sums over each expert's kept rows: out[e, c] = sum_{rows p of e} src[p, c]
 // (d_down_proj_bias and d_gate_up_proj_bias, csrc/experts_backward.cu:277, 308).
-// grid (E, ceil(cols / kRowThreads)); a thread owns one column and walks the rows in order.
+// grid (E, ceil(cols / (64 * V))), V = elements per 16 bytes: a workgroup owns one expert and 64 * V columns,
+// its waves take every kRowWaves-th row with 16 bytes per lane (eight rows in flight per wave), and the
+// per-wave partial sums meet in LDS.  The order of the additions is fixed, so the result is reproducible.
 template <typename T>
 __global__ __launch_bounds__(kRowThreads) void expert_colsum_kernel(const T *__restrict__ src,
                                                                     const int *__restrict__ counts,
                                                                     const int *__restrict__ offsets,
                                                                     int capacity, T *__restrict__ out,
                                                                     int cols) {
+  constexpr int V = ElemTraits<T>::kVec;
+  __shared__ float part[kRowWaves][kWave * V];
+  const int e = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c0 = (blockIdx.y * kWave + lane) * V;
+  const int first = offsets[e], kept = min(counts[e], capacity);
+  float acc[V];
+#pragma unroll
+  for (int v = 0; v < V; ++v) acc[v] = 0.0f;
+  if (c0 < cols) {
+    const T *p = src + (size_t)first * cols + c0;
+    auto add = [&](const u32x4 &raw) {
+      const T *h = (const T *)&raw;
+#pragma unroll
+      for (int v = 0; v < V; ++v) acc[v] += ElemTraits<T>::to_f32(h[v]);
+    };
+    int r = wave;
+    for (; r + 7 * kRowWaves < kept; r += 8 * kRowWaves) {
+      u32x4 raw[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) raw[j] = *(const u32x4 *)(p + (size_t)(r + j * kRowWaves) * cols);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) add(raw[j]);
+    }
+    for (; r < kept; r += kRowWaves) add(*(const u32x4 *)(p + (size_t)r * cols));
+  }
+#pragma unroll
+  for (int v = 0; v < V; ++v) part[wave][lane * V + v] = acc[v];
+  __syncthreads();
+  for (int i = threadIdx.x; i < kWave * V; i += kRowThreads) {
+    int c = blockIdx.y * kWave * V + i;
+    if (c < cols) {
+      float sum = 0.0f;
+#pragma unroll
+      for (int w = 0; w < kRowWaves; ++w) sum += part[w][i];
+      out[(size_t)e * cols + c] = ElemTraits<T>::from_f32(sum);
+    }
+  }
+}
+
+// the same for a column count that is not a multiple of the 16-byte vector: a thread per column
+template <typename T>
+__global__ __launch_bounds__(kRowThreads) void expert_colsum_scalar_kernel(const T *__restrict__ src,
+                                                                           const int *__restrict__ counts,
+                                                                           const int *__restrict__ offsets,
+                                                                           int capacity, T *__restrict__ out,
+                                                                           int cols) {
   const int e = blockIdx.x;
   const int c = blockIdx.y * kRowThreads + threadIdx.x;
   if (c >= cols) return;
@@ -212,8 +260,13 @@ int launch_combine_backward(const void *grad_out, const void *y_perm, const int 
 template <typename T>
 int launch_expert_colsum(const void *src, const int *counts, const int *offsets, int capacity,
                          void *out, int E, int cols, hipStream_t stream) {
-  hipLaunchKernelGGL(expert_colsum_kernel<T>, dim3(E, ceil_div(cols, kRowThreads)), dim3(kRowThreads), 0,
-                     stream, (const T *)src, counts, offsets, capacity, (T *)out, cols);
+  constexpr int V = ElemTraits<T>::kVec;
+  if (cols % V == 0)
+    hipLaunchKernelGGL(expert_colsum_kernel<T>, dim3(E, ceil_div(cols, kWave * V)), dim3(kRowThreads), 0, stream,
+                       (const T *)src, counts, offsets, capacity, (T *)out, cols);
+  else
+    hipLaunchKernelGGL(expert_colsum_scalar_kernel<T>, dim3(E, ceil_div(cols, kRowThreads)), dim3(kRowThreads), 0,
+                       stream, (const T *)src, counts, offsets, capacity, (T *)out, cols);
   return check_launch("expert_colsum_kernel");
 }
 
