@@ -59,7 +59,10 @@ template <typename T>
 int gemm_async_down(const void *, const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);
 template <typename T>
 int gemm_async_dgrad(const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);
+template <typename T>
+int gemm_async_wgrad(const void *, const void *, void *, const int *, const int *, int, int, int, int, hipStream_t);
 bool gemm_async_supported(int Kd, int Nd, int lda, int ldb, long long a_span_bytes);
+bool wgrad_async_supported(int Md, int Nd);
 
 template <typename T> struct HasStreamPath { static constexpr bool value = sizeof(T) == 2; };
 
@@ -91,6 +94,15 @@ static int tiles_dgrad(const void *g, const void *w, void *out, const void *sche
     if (gemm_async_supported(Kd, Nd, Kd, Kd, 0)) return gemm_async_dgrad<T>(g, w, out, sched, N, E, Kd, Nd, stream);
   }
   return gemm_dgrad<T>(g, w, out, sched, N, E, Kd, Nd, stream);
+}
+
+template <typename T>
+static int tiles_wgrad(const void *L, const void *R, void *dW, const int *counts, const int *offsets, int capacity, int E,
+                       int Md, int Nd, hipStream_t stream) {
+  if constexpr (sizeof(T) == 2) {
+    if (wgrad_async_supported(Md, Nd)) return gemm_async_wgrad<T>(L, R, dW, counts, offsets, capacity, E, Md, Nd, stream);
+  }
+  return gemm_wgrad<T>(L, R, dW, counts, offsets, capacity, E, Md, Nd, stream);
 }
 
 __global__ void fill_zero_kernel(uint32_t *p, long long n_words) {
@@ -185,6 +197,10 @@ static size_t carve_backward(const yamoe_problem *p, void *ws, BackwardBuffers *
   // d_act [N, I] reuses the y_perm region (dead after the combine backward)
   b->d_act = b->f.y_perm;
   b->d_x_perm = c.take(N * p->H * es);
+  // the weight-gradient kernel's copies of an expert's last, partial slab of rows run up to 32 rows past the
+  // end of its operand buffers; every operand is followed by another buffer of this workspace, and this pad
+  // covers the case where those are smaller than 32 rows of the widest operand
+  c.take(32 * (size_t)(p->H > 2 * p->I ? p->H : 2 * p->I) * es);
   return used + c.used;
 }
 
@@ -249,13 +265,13 @@ static int backward_impl(const yamoe_problem *p, const void *gy, const void *x, 
   // down projection
   YAMOE_TRY(launch_expert_colsum<T>(b.g_y_perm, b.f.counts, b.f.offsets, cap, d_bd, E, H, stream));
   YAMOE_TRY(tiles_dgrad<T>(b.g_y_perm, wd, b.d_act, b.f.schedule, N, E, /*Kd=*/H, /*Nd=*/I, stream));
-  YAMOE_TRY(gemm_wgrad<T>(b.f.act, b.g_y_perm, d_wd, b.f.counts, b.f.offsets, cap, E, /*Md=*/I, /*Nd=*/H, stream));
+  YAMOE_TRY(tiles_wgrad<T>(b.f.act, b.g_y_perm, d_wd, b.f.counts, b.f.offsets, cap, E, /*Md=*/I, /*Nd=*/H, stream));
   // GLU
   YAMOE_TRY(glu_backward_rows<T>(b.d_act, b.pre, b.d_pre, (long long)N * I, stream));
   // gate_up projection
   YAMOE_TRY(launch_expert_colsum<T>(b.d_pre, b.f.counts, b.f.offsets, cap, d_bgu, E, 2 * I, stream));
   YAMOE_TRY(tiles_dgrad<T>(b.d_pre, wgu, b.d_x_perm, b.f.schedule, N, E, /*Kd=*/2 * I, /*Nd=*/H, stream));
-  YAMOE_TRY(gemm_wgrad<T>(b.x_perm, b.d_pre, d_wgu, b.f.counts, b.f.offsets, cap, E, /*Md=*/H, /*Nd=*/2 * I, stream));
+  YAMOE_TRY(tiles_wgrad<T>(b.x_perm, b.d_pre, d_wgu, b.f.counts, b.f.offsets, cap, E, /*Md=*/H, /*Nd=*/2 * I, stream));
   // permute backward: d_hidden[t] = sum_k d_x_perm[inv_pos[t,k]]
   YAMOE_TRY(launch_combine<T>(b.d_x_perm, b.f.inv_pos, idx, p->idx_i64, nullptr, p->K, d_x, p->T, p->K, E, H, stream));
   return 0;

@@ -514,6 +514,259 @@ static int launch(const Args &args, int max_row_tiles, hipStream_t stream) {
   return check_launch("gemm_async_kernel");
 }
 
+
+// ---- weight gradients: dW[e] = L[rows of e]^T * R[rows of e] -----------------------------------------------
+// (csrc/experts_backward.cu:198, 311).  The contraction runs over the expert's kept rows, so both operands are
+// [k][m] / [k][n] in memory: both stay that way in LDS (4 + 4 single-slab buffers of 32 k-rows x 512 bytes)
+// and both are read with the LDS transpose read.  The last slab of an expert is usually partial: the copies
+// of its missing rows read whatever follows in memory (the caller keeps that readable) and the wave that
+// issued them overwrites them with zeros in LDS before anybody reads the slab.
+struct WgradArgs {
+  const void *A;  // [N, Md] rows in expert order
+  const void *B;  // [N, Nd]
+  void *C;        // [E, Md, Nd]
+  const int *counts, *offsets;
+  int capacity, E, Md, Nd, n_m_tiles, n_n_tiles;
+};
+
+template <bool P1_, bool P2_, bool NEXT_, bool ZERO_, int VM_> struct WStepCfg {
+  static constexpr bool P1 = P1_, P2 = P2_, NEXT = NEXT_, ZERO = ZERO_;
+  static constexpr int VM = VM_;
+};
+
+template <typename T, int NMI>
+__device__ inline void run_wgrad_tile(const WgradArgs &args, const int tid, const int expert, const int m0, const int n0,
+                                      const int rows_m, const long long first, const int rows) {
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  constexpr int NACC = NMI > 0 ? NMI : 1;
+  constexpr int kStage = 16384, kARing = 0, kBRing2 = 4 * kStage;
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds);
+
+  f32x16 acc[NACC][4];
+#pragma unroll
+  for (int mi = 0; mi < NACC; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < 4; ++ni)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
+
+  const int n_slabs = (rows + kBK - 1) / kBK;
+  const long long lda_bytes = (long long)args.Md * (long long)sizeof(T), ldb_bytes = (long long)args.Nd * (long long)sizeof(T);
+
+  // copies: piece i (0..3) of a slab = k rows 8*wave + 2*i + (lane >> 5); LDS position lane & 31 holds piece
+  // pos ^ ((k & 3) << 2) of the 512-byte row
+  uint32_t a_off[4], b_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int k = 8 * wave + 2 * i + (lane >> 5);
+    int piece = (lane & 31) ^ ((k & 3) << 2);
+    int ca = m0 + piece * 8, cb = n0 + piece * 8;
+    if (ca >= args.Md) ca = m0;  // columns past the end re-read valid ones; never stored
+    if (cb >= args.Nd) cb = n0;
+    a_off[i] = (uint32_t)(k * lda_bytes + (long long)(ca - m0) * (long long)sizeof(T));
+    b_off[i] = (uint32_t)(k * ldb_bytes + (long long)(cb - n0) * (long long)sizeof(T));
+  }
+  const char *a_base = (const char *)((const T *)args.A + first * args.Md + m0);
+  const char *b_base = (const char *)((const T *)args.B + first * args.Nd + n0);
+  auto copy_a = [&](int slab, int i) {
+    copy16_to_lds(a_base + (long long)slab * kBK * lda_bytes, a_off[i],
+                  lds0 + kARing + (uint32_t)(slab & 3) * kStage + (uint32_t)(8 * wave + 2 * i) * 512u);
+  };
+  auto copy_b = [&](int slab, int i) {
+    copy16_to_lds(b_base + (long long)slab * kBK * ldb_bytes, b_off[i],
+                  lds0 + kBRing2 + (uint32_t)(slab & 3) * kStage + (uint32_t)(8 * wave + 2 * i) * 512u);
+  };
+  // rows of slab `slab` at or past the end of the expert become zeros (this wave's own pieces, which have landed)
+  auto zero_tail = [&](int slab) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int k = 8 * wave + 2 * i + (lane >> 5);
+      if (slab * kBK + k >= rows) {
+        const int o = (slab & 3) * kStage + (8 * wave + 2 * i) * 512 + lane * 16;
+        *(u32x4 *)(lds + kARing + o) = (u32x4){0, 0, 0, 0};
+        *(u32x4 *)(lds + kBRing2 + o) = (u32x4){0, 0, 0, 0};
+      }
+    }
+  };
+
+  // operand reads: k = ks*16 + g*8 + h*4 + j, 4 columns at c + 16*((lane>>4)&1) + 4*q with j = (lane&15)>>2, q = lane&3
+  const int g = lane >> 5, rl = lane & 31, j4 = (lane & 15) >> 2, q4 = lane & 3;
+  int a_rd[NACC], b_rd[4];
+#pragma unroll
+  for (int mi = 0; mi < NACC; ++mi) {
+    int col = (mi * 2 + wm) * 32 + 16 * ((lane >> 4) & 1) + 4 * q4;
+    a_rd[mi] = (g * 8 + j4) * 512 + ((((col >> 3) ^ (j4 << 2))) << 4) + (col & 7) * 2;
+  }
+#pragma unroll
+  for (int ni = 0; ni < 4; ++ni) {
+    int col = wn * 128 + ni * 32 + 16 * ((lane >> 4) & 1) + 4 * q4;
+    b_rd[ni] = (g * 8 + j4) * 512 + ((((col >> 3) ^ (j4 << 2))) << 4) + (col & 7) * 2;
+  }
+  u32x4 fa0[NACC], fa1[NACC], fb0[4], fb1[4];
+  constexpr int kFrags = NMI > 0 ? 4 + NMI : 0;
+  // fragment order B0, A0, B1, B2, B3, A1, A2, A3
+  auto read_frag = [&](int s, int ks, int f, u32x4 (&fa)[NACC], u32x4 (&fb)[4]) {
+    const bool is_a = f == 1 || f >= 5;
+    const int idx = is_a ? (f == 1 ? 0 : f - 4) : (f == 0 ? 0 : f - 1);
+    const char *sp = lds + (is_a ? kARing : kBRing2) + (s & 3) * kStage + (is_a ? a_rd[idx] : b_rd[idx]) + ks * 8192;
+    u32x2 lo = lds_read_tr16(sp);
+    u32x2 hi = lds_read_tr16(sp + 2048);
+    u32x4 v = (u32x4){lo[0], lo[1], hi[0], hi[1]};
+    if (is_a) fa[idx] = v; else fb[idx] = v;
+  };
+  auto read_frags = [&](int s, int ks, u32x4 (&fa)[NACC], u32x4 (&fb)[4]) {
+#pragma unroll
+    for (int f = 0; f < kFrags; ++f) read_frag(s, ks, f, fa, fb);
+  };
+
+  // ---- pipeline: as in run_tile, with both operands on single-slab rings ------------------------------------------
+  //   second k-step of slab t: first halves (2 + 2 copies) of slab t + 4;  first k-step of slab t + 1: second halves
+  // i.e. 4 copies per wave in every k-step, and "slab s+1 has landed" means at most 16 younger copies in flight.
+  constexpr int kMma = 4 * NMI;
+  constexpr int kSlots = kMma > 2 ? kMma - 2 : 1;
+  if (n_slabs > 0) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+      if (s < n_slabs) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { copy_a(s, i); copy_b(s, i); }
+      }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+      if (s < n_slabs && (s + 1) * kBK > rows) zero_tail(s);
+    __syncthreads();
+    read_frags(0, 0, fa0, fb0);
+  }
+  auto slab_step = [&](int s, auto cfg) {
+    typedef decltype(cfg) C;
+    __builtin_amdgcn_sched_barrier(0);
+    {
+      constexpr int kC = C::P1 ? 4 : 0, kItems = kC + kFrags;
+#pragma unroll
+      for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
+        if (j < kMma) Mma<T>::run(fa0[j >> 2], fb0[j & 3], acc[j >> 2][j & 3]);
+        if (j < kSlots) {
+#pragma unroll
+          for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
+            if (i < kC) { if (i < 2) copy_a(s + 3, 2 + i); else copy_b(s + 3, i); }
+            else read_frag(s, 1, i - kC, fa1, fb1);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    if constexpr (C::VM == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else if constexpr (C::VM == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else if constexpr (C::VM == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if constexpr (C::ZERO) zero_tail(s + 1);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    {
+      constexpr int kC = C::P2 ? 4 : 0, kItems = kC + (C::NEXT ? kFrags : 0);
+#pragma unroll
+      for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
+        if (j < kMma) Mma<T>::run(fa1[j >> 2], fb1[j & 3], acc[j >> 2][j & 3]);
+        if (j < kSlots) {
+#pragma unroll
+          for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
+            if (i < kC) { if (i < 2) copy_a(s + 4, i); else copy_b(s + 4, i - 2); }
+            else read_frag(s + 1, 0, i - kC, fa0, fb0);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+  if (n_slabs >= 8) {
+    slab_step(0, WStepCfg<false, true, true, false, -1>());
+    int s = 1;
+    for (; s + 5 < n_slabs; ++s) slab_step(s, WStepCfg<true, true, true, false, 16>());
+    // s = n_slabs - 5: the last copies (second halves of slab n_slabs - 1) go out in the first k-step of slab n_slabs - 4
+    slab_step(s, WStepCfg<true, true, true, false, 16>());
+    slab_step(s + 1, WStepCfg<true, false, true, false, 16>());
+    slab_step(s + 2, WStepCfg<false, false, true, false, 8>());
+    slab_step(s + 3, WStepCfg<false, false, true, true, 0>());
+    slab_step(s + 4, WStepCfg<false, false, false, false, -1>());
+  } else {
+    for (int s = 0; s < n_slabs; ++s) {
+      if (kFrags > 0) read_frags(s, 1, fa1, fb1);
+#pragma unroll
+      for (int j = 0; j < kMma; ++j) Mma<T>::run(fa0[j >> 2], fb0[j & 3], acc[j >> 2][j & 3]);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (s + 1 < n_slabs && (s + 2) * kBK > rows) zero_tail(s + 1);
+      __syncthreads();
+      if (s + 4 < n_slabs) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { copy_a(s + 4, i); copy_b(s + 4, i); }
+      }
+      if (s + 1 < n_slabs) read_frags(s + 1, 0, fa0, fb0);
+#pragma unroll
+      for (int j = 0; j < kMma; ++j) Mma<T>::run(fa1[j >> 2], fb1[j & 3], acc[j >> 2][j & 3]);
+    }
+  }
+
+  // ---- epilogue: stage the tile in LDS, store whole row segments ------------------------------------------------
+  constexpr int stride = kBN * 2 + 16;
+  const int rsub = g * 4;
+  __syncthreads();
+  {
+    char *lp0 = lds + (wm * 32 + rsub) * stride + (wn * 128 + rl) * 2;
+    char *lp1 = lp0 + 128 * stride;
+#pragma unroll
+    for (int ni = 0; ni < 4; ++ni)
+#pragma unroll
+      for (int mi = 0; mi < NMI; ++mi)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          char *q = (mi < 2 ? lp0 : lp1) + ((mi & 1) * 64 + 8 * (v >> 2) + (v & 3)) * stride + ni * 64;
+          *(T *)q = ElemTraits<T>::from_f32(acc[mi][ni][v]);
+        }
+  }
+  __syncthreads();
+  {
+    constexpr int chunks = kBN >> 3, rows_per_pass = kThreads / chunks;
+    const int c = tid % chunks;
+    if (n0 + c * 8 < args.Nd) {
+      T *p = (T *)args.C + ((long long)expert * args.Md + m0) * args.Nd + n0 + c * 8;
+      for (int r = tid / chunks; r < rows_m; r += rows_per_pass)
+        *(u32x4 *)(p + (long long)r * args.Nd) = *(const u32x4 *)(lds + r * stride + c * 16);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void wgrad_async_kernel(const WgradArgs args) {
+  const int tid = threadIdx.x, wave = tid >> 6, wm = wave >> 1;
+  // tile list: expert, then column tile, then row tiles; workgroup b runs on XCD b % 8, which takes a contiguous
+  // eighth of the list
+  const int per_expert = args.n_m_tiles * args.n_n_tiles;
+  const int total = args.E * per_expert;
+  const int total8 = (total + kXcds - 1) / kXcds * kXcds;
+  const int b = blockIdx.x;
+  if (b >= total8) return;
+  const int L = (b % kXcds) * (total8 / kXcds) + b / kXcds;
+  if (L >= total) return;
+  const int expert = L / per_expert, r = L - expert * per_expert;
+  const int n0 = (r / args.n_m_tiles) * kBN, m0 = (r % args.n_m_tiles) * kBM;
+  const int rows_m = min(kBM, args.Md - m0);
+  int rows = min(args.counts[expert], args.capacity);
+  if (rows < 0) rows = 0;
+  const long long first = args.offsets[expert];
+  const int n_blocks32 = (rows_m + 31) >> 5;
+  const int n_mi = (n_blocks32 - wm + 1) >> 1;
+  switch (n_mi) {
+    case 4: run_wgrad_tile<T, 4>(args, tid, expert, m0, n0, rows_m, first, rows); break;
+    case 3: run_wgrad_tile<T, 3>(args, tid, expert, m0, n0, rows_m, first, rows); break;
+    case 2: run_wgrad_tile<T, 2>(args, tid, expert, m0, n0, rows_m, first, rows); break;
+    case 1: run_wgrad_tile<T, 1>(args, tid, expert, m0, n0, rows_m, first, rows); break;
+    default: run_wgrad_tile<T, 0>(args, tid, expert, m0, n0, rows_m, first, rows); break;
+  }
+}
+
 }  // namespace async
 
 // True when the asynchronous-copy kernels can take this product.
@@ -558,12 +811,43 @@ int gemm_async_dgrad(const void *g, const void *w, void *out, const void *sched,
   return async::launch<T, async::EPI_STORE, false, true>(a, sched_max_row_tiles(N, E), stream);
 }
 
+// dW[E, Md, Nd] = per expert L^T R over its kept rows.  Both operand buffers must stay readable for 32 rows past
+// their last row (the copies of a partial last slab run over; what they fetch is zeroed before use).
+bool wgrad_async_supported(int Md, int Nd) { return Md % 8 == 0 && Nd % 8 == 0; }
+
+template <typename T>
+int gemm_async_wgrad(const void *L, const void *R, void *dW, const int *counts, const int *offsets, int capacity, int E,
+                     int Md, int Nd, hipStream_t stream) {
+  async::WgradArgs a = {};
+  a.A = L; a.B = R; a.C = dW; a.counts = counts; a.offsets = offsets; a.capacity = capacity;
+  a.E = E; a.Md = Md; a.Nd = Nd;
+  a.n_m_tiles = ceil_div(Md, async::kBM);
+  a.n_n_tiles = ceil_div(Nd, async::kBN);
+  auto kernel = async::wgrad_async_kernel<T>;
+  static bool attr_done = false;  // benign race: the attribute call is idempotent
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, async::kLds);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(MaxDynamicSharedMemorySize=%d): %s", async::kLds, hipGetErrorString(e));
+      return (int)e;
+    }
+    attr_done = true;
+  }
+  long long total = (long long)E * a.n_m_tiles * a.n_n_tiles;
+  if (total <= 0) return 0;
+  total = (total + kXcds - 1) / kXcds * kXcds;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(async::kThreads), async::kLds, stream, a);
+  return check_launch("wgrad_async_kernel");
+}
+
 #define YAMOE_INSTANTIATE_ASYNC(T)                                                                               \
   template int gemm_async_gate_up<T>(const void *, const int *, const void *, const void *, void *, void *,      \
                                      const void *, int, int, int, int, int, hipStream_t);                        \
   template int gemm_async_down<T>(const void *, const void *, const void *, void *, const void *, int, int, int, \
                                   int, hipStream_t);                                                             \
-  template int gemm_async_dgrad<T>(const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);
+  template int gemm_async_dgrad<T>(const void *, const void *, void *, const void *, int, int, int, int, hipStream_t); \
+  template int gemm_async_wgrad<T>(const void *, const void *, void *, const int *, const int *, int, int, int, int,    \
+                                   hipStream_t);
 YAMOE_INSTANTIATE_ASYNC(bf16_t)
 YAMOE_INSTANTIATE_ASYNC(f16_t)
 
