@@ -180,6 +180,17 @@ int yamoe_batch_mm(const void *x, const void *weights, void *output, int32_t E, 
                    int32_t Kd, int32_t Nd, int32_t dtype, void *workspace, size_t workspace_bytes,
                    void *stream);
 
+/* The router step of Yamoe.forward (torch-ext/yamoe/layers.py:128-152; GptOssTopKRouter.forward,
+ * torch-ext/yamoe/vendored/gpt_oss_mlp.py:128-142) in one kernel, 16-bit dtypes:
+ *   logits = round(hidden . weight^T + bias)            [T,E]  (optional output)
+ *   router_indices = top_k experts by logit, descending; equal logits: lower expert id first   [T,K] int64
+ *   router_scores  = softmax over the K picked logits (fp32, rounded once), scattered into a
+ *                    zero [T,E] row; topk_weights (optional) holds the same K values as [T,K].
+ * H must be a multiple of 16, E <= 256, top_k <= min(E, 16).  bias may be NULL. */
+int yamoe_router_topk(const void *hidden, const void *weight, const void *bias, int32_t T, int32_t H,
+                      int32_t E, int32_t top_k, int32_t dtype, int64_t *router_indices,
+                      void *router_scores, void *topk_weights, void *logits, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

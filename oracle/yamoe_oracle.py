@@ -31,6 +31,9 @@ formula under test):
                         must reproduce experts_capacity, which is pinned on its own above; padding
                         rows must be zero; gather followed by unweighted scatter multiplies each
                         token row by its number of kept slots
+  router                brute-force Python top-k with the same tie rule on small inputs, torch.topk values
+                        (a library routine; values agree whatever its tie order), rows of scores sum to 1 and
+                        are zero off the selection
 The reference ships no golden vectors or known-answer tests for this path (its tests directory is
 git-ignored), so no reference-held fixture exists to check against; no function here is
 "parity unpinned" in the sense of lacking an independent check.
@@ -311,6 +314,32 @@ def batch_mm(x, weights, compute_dtype=torch.float64):
     """Per-expert product [E, C, K] x [E, K, N]; batch_sizes and trans_b are not used by the
     reference (csrc/batch_mm.cu:7-31 is one bmm)."""
     return torch.bmm(x.to(compute_dtype), weights.to(compute_dtype))
+
+
+# ------------------------------------------------------------------------------------------------
+# router step
+# ------------------------------------------------------------------------------------------------
+def router_from_logits(logits, top_k):
+    """top-k -> softmax over the picked logits -> dense scores (torch-ext/yamoe/layers.py:135-152,
+    torch-ext/yamoe/vendored/gpt_oss_mlp.py:134-142).  Picks come in descending order of logit; among equal
+    logits the lower expert id first (torch.topk leaves that order open).  The softmax is taken in fp32 and
+    rounded once to the logits' dtype.  Returns (router_indices int64 [T,K], router_scores [T,E])."""
+    order = torch.sort(logits.float(), dim=-1, descending=True, stable=True).indices[:, :top_k]
+    top = torch.gather(logits.float(), 1, order)
+    w = torch.softmax(top, dim=-1).to(logits.dtype)
+    scores = torch.zeros_like(logits).scatter_(1, order, w)
+    return order, scores
+
+
+def router(hidden, weight, bias, top_k):
+    """logits = hidden . weight^T + bias in fp32, rounded to the activation dtype (the output of the reference's
+    F.linear, layers.py:130-132), then router_from_logits.  Returns (indices, scores, logits)."""
+    logits = hidden.float() @ weight.float().t()
+    if bias is not None:
+        logits = logits + bias.float()
+    logits = logits.to(hidden.dtype)
+    idx, scores = router_from_logits(logits, top_k)
+    return idx, scores, logits
 
 
 def rel_l2(a, b):

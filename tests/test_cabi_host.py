@@ -76,6 +76,7 @@ def test_torch_op_schemas_match_reference():
     assert schema("index_select_out") == "index_select_out(Tensor! out, Tensor input, Tensor idx_int32) -> Tensor"
     assert schema("batch_mm") == ("batch_mm(Tensor x, Tensor weights, Tensor batch_sizes, Tensor! output, "
                                   "bool trans_b=False) -> Tensor")
+    assert schema("router_topk") == "router_topk(Tensor hidden, Tensor weight, Tensor? bias, int top_k) -> (Tensor, Tensor)"
     for name in ("gather", "scatter", "sort", "bincount_cumsum", "batch_mm", "experts", "experts_backward", "Yamoe"):
         assert getattr(yamoe_amd, name) is not None       # the reference package's exports (torch-ext/yamoe/__init__.py)
 

@@ -1,0 +1,108 @@
+"""The fused router step (linear -> top-k -> softmax -> dense scores) against the oracle, and the Yamoe layer
+built on it (torch-ext/yamoe/layers.py:106-218)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import yamoe_oracle as O
+from tests.util import REL_L2_TOL, report
+
+pytestmark = pytest.mark.gpu
+
+
+def draw(T, H, E, dtype, seed, bias=True):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    w = (torch.randn(E, H, generator=g) / H ** 0.5 * 2).to(dtype)
+    b = torch.randn(E, generator=g).to(dtype) if bias else None
+    return x, w, b
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,H,E,K", [(4096, 2880, 32, 4), (64, 2880, 128, 4), (1, 64, 8, 2), (77, 128, 5, 5), (300, 256, 200, 16),
+                                     (33, 48, 33, 1)])
+def test_router_topk(gpu, dtype, T, H, E, K):
+    from yamoe_amd import _cabi
+    print("router", dtype, T, H, E, K, flush=True)
+    x, w, b = draw(T, H, E, dtype, T + E, bias=(E != 5))
+    idx, scores, topw, logits = _cabi.router_topk(x.to(gpu), w.to(gpu), None if b is None else b.to(gpu), K)
+    torch.cuda.synchronize()
+    idx, scores, topw, logits = idx.cpu(), scores.cpu(), topw.cpu(), logits.cpu()
+    # the linear: fp32 accumulation in another order than the oracle's, so a logit may land one rounding step away
+    _, _, want_logits = O.router(x, w, b, K)
+    ulp = 2.0 ** (-7 if dtype == torch.bfloat16 else -10)
+    diff = (logits.float() - want_logits.float()).abs()
+    assert torch.all(diff <= ulp * torch.maximum(want_logits.float().abs(), torch.full_like(diff, 2.0 ** -6)) + 1e-6)
+    assert (diff > 0).float().mean() < 0.05
+    # top-k, softmax and scatter on the kernel's own logits: picks bit-exact (ties included), weights within one rounding step
+    want_idx, want_scores = O.router_from_logits(logits, K)
+    assert torch.equal(idx, want_idx)
+    assert torch.all((scores.float() - want_scores.float()).abs() <= ulp * want_scores.float())
+    assert (scores != want_scores).float().mean() < 0.01
+    assert torch.equal(torch.gather(scores, 1, idx), topw)
+    assert torch.equal(scores != 0, torch.zeros_like(scores, dtype=torch.bool).scatter_(1, idx, topw != 0))
+
+
+def test_router_ties_pick_lower_expert(gpu):
+    from yamoe_amd import _cabi
+    # identical weight rows give identical logits: the pick order must be by expert id
+    T, H, E, K = 40, 64, 16, 4
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    w = torch.randn(1, H, generator=g).to(torch.bfloat16).repeat(E, 1)
+    idx, scores, topw, logits = _cabi.router_topk(x.to(gpu), w.to(gpu), None, K)
+    torch.cuda.synchronize()
+    assert torch.equal(idx.cpu(), torch.arange(K).repeat(T, 1))
+    assert torch.all(topw.cpu().float() == 0.25)
+
+
+def test_router_rejects(gpu):
+    import yamoe_amd
+    x, w, b = draw(8, 64, 4, torch.bfloat16, 0)
+    with pytest.raises(RuntimeError):
+        yamoe_amd.router_topk(x.float().to(gpu), w.float().to(gpu), b.float().to(gpu), 2)      # fp32: not taken
+    with pytest.raises(RuntimeError):
+        yamoe_amd.router_topk(x.to(gpu), w.to(gpu), b.to(gpu), 5)                               # top_k > E
+    with pytest.raises(RuntimeError):
+        yamoe_amd.router_topk(x[:, :40].contiguous().to(gpu), w[:, :40].contiguous().to(gpu), b.to(gpu), 2)  # H % 16
+
+
+class Block(torch.nn.Module):
+    """The attributes Yamoe.forward expects from its host module."""
+
+    def __init__(self, H, I, E, K, dtype, seed):
+        super().__init__()
+        g = torch.Generator().manual_seed(seed)
+
+        def p(*shape, std=0.05):
+            return torch.nn.Parameter((torch.randn(*shape, generator=g) * std).to(dtype))
+        self.router = torch.nn.Module()
+        self.router.weight, self.router.bias = p(E, H, std=0.2), p(E, std=0.5)
+        self.experts = torch.nn.Module()
+        self.experts.gate_up_proj, self.experts.gate_up_proj_bias = p(E, H, 2 * I), p(E, 2 * I, std=0.1)
+        self.experts.down_proj, self.experts.down_proj_bias = p(E, I, H), p(E, H, std=0.1)
+        self.num_experts, self.top_k = E, K
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_yamoe_layer_forward(gpu, dtype):
+    import yamoe_amd
+    B, S, H, I, E, K = 2, 96, 128, 64, 8, 2
+    blk = Block(H, I, E, K, dtype, 4)
+    x = torch.randn(B, S, H, generator=torch.Generator().manual_seed(5)).to(dtype)
+    dev = Block(H, I, E, K, dtype, 4).to(gpu)
+    with torch.no_grad():
+        out, scores = yamoe_amd.Yamoe.forward(dev, x.to(gpu))
+    torch.cuda.synchronize()
+    out, scores = out.cpu(), scores.cpu()
+    assert out.shape == (B, S, H) and scores.shape == (B * S, E)
+    # router: a logit one rounding step away may swap two near-equal experts, so compare what survives that: the
+    # scores as a whole, then the expert layer on the layer's own routing
+    _, want_scores, _ = O.router(x.reshape(-1, H), blk.router.weight.data, blk.router.bias.data, K)
+    assert report("router scores", scores.double(), want_scores.double(), 3e-2) < 3e-2
+    idx = torch.topk(scores.float(), K, dim=-1).indices
+    want = O.experts_capacity(x.reshape(-1, H), idx, scores, blk.experts.gate_up_proj.data, blk.experts.gate_up_proj_bias.data,
+                              blk.experts.down_proj.data, blk.experts.down_proj_bias.data, B * S, compute_dtype=torch.float64)
+    tol = REL_L2_TOL[dtype]
+    assert report("layer", out.reshape(-1, H).double(), want, tol) < tol
+    assert (scores != 0).sum(-1).max() <= K

@@ -2,6 +2,7 @@
 brute force, library routines, closed-form special cases, finite differences and a hand-made
 known-answer fixture.  The reference ships no fixtures for this path, so these are the anchors."""
 import json
+import math
 import os
 
 import numpy as np
@@ -296,3 +297,44 @@ def test_gather_then_plain_scatter_counts_kept_slots():
             kept[f // K] += 1
     want = y0 + d["hidden"] * torch.from_numpy(kept)[:, None]
     assert O.rel_l2(out, want) < 1e-14
+
+
+# ---- router step -----------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_router_from_logits_brute_force(dtype):
+    g = torch.Generator().manual_seed(9)
+    T, E, K = 50, 12, 4
+    logits = (torch.randn(T, E, generator=g) * 2).to(dtype)
+    logits[:, 3] = logits[:, 7]                       # ties in every row
+    logits[5] = 0.25                                  # a row of all-equal logits: picks 0, 1, 2, 3
+    idx, scores = O.router_from_logits(logits, K)
+    for t in range(T):
+        row = [float(v) for v in logits[t]]
+        picked = []
+        for _ in range(K):
+            best = None
+            for e in range(E):
+                if e not in picked and (best is None or row[e] > row[best]):
+                    best = e
+            picked.append(best)
+        assert idx[t].tolist() == picked
+        ex = [math.exp(row[e] - row[picked[0]]) for e in picked]
+        for k, e in enumerate(picked):
+            want = torch.tensor(ex[k] / sum(ex), dtype=torch.float64).to(dtype)
+            assert abs(float(scores[t, e]) - float(want)) <= (2 ** -8 if dtype == torch.bfloat16 else 1e-6) * float(want)
+        off = [e for e in range(E) if e not in picked]
+        assert all(float(scores[t, e]) == 0.0 for e in off)
+    vals = torch.topk(logits.float(), K, dim=-1).values
+    assert torch.equal(torch.gather(logits.float(), 1, idx), vals)
+    assert torch.allclose(scores.float().sum(-1), torch.ones(T), atol=2e-2 if dtype == torch.bfloat16 else 1e-6)
+
+
+def test_router_linear_rounds_once():
+    g = torch.Generator().manual_seed(10)
+    x = torch.randn(7, 32, generator=g).to(torch.bfloat16)
+    w = torch.randn(5, 32, generator=g).to(torch.bfloat16)
+    b = torch.randn(5, generator=g).to(torch.bfloat16)
+    idx, scores, logits = O.router(x, w, b, 2)
+    want = (x.double() @ w.double().t() + b.double()).to(torch.bfloat16)
+    assert logits.dtype == torch.bfloat16 and (logits.float() - want.float()).abs().max() <= 2 ** -7 * want.float().abs().max()
+    assert idx.shape == (7, 2) and scores.shape == (7, 5)

@@ -4,7 +4,8 @@ Same surface as the reference package for this path (torch-ext/yamoe/__init__.py
 `experts`, `experts_backward`, `gather`, `scatter`, `sort`, `bincount_cumsum`, `batch_mm`, `ops`, `Yamoe`.  Everything runs in hand-written HIP kernels behind
 the C ABI of libyamoe_hip.so; the first use of any of them fails if the native libraries are not built.
 """
-_OPS = ("gather", "scatter", "sort", "bincount_cumsum", "index_select_out", "batch_mm", "experts", "experts_backward")
+_OPS = ("gather", "scatter", "sort", "bincount_cumsum", "index_select_out", "batch_mm", "experts", "experts_backward",
+        "router_topk")
 _LAYERS = ("Yamoe", "experts_autograd")
 
 __all__ = ["ops", *_LAYERS, *_OPS]

@@ -22,7 +22,7 @@ SYMBOLS = [
     "yamoe_experts_workspace_bytes", "yamoe_experts_forward", "yamoe_experts_backward_workspace_bytes",
     "yamoe_experts_backward", "yamoe_sort_workspace_bytes", "yamoe_sort", "yamoe_bincount_cumsum", "yamoe_padded_gather",
     "yamoe_padded_scatter_workspace_bytes", "yamoe_padded_scatter", "yamoe_index_select", "yamoe_regular_groups",
-    "yamoe_batch_mm_workspace_bytes", "yamoe_batch_mm",
+    "yamoe_batch_mm_workspace_bytes", "yamoe_batch_mm", "yamoe_router_topk",
 ]
 
 
@@ -59,6 +59,7 @@ def lib():
         L.yamoe_experts_backward_workspace_bytes.restype = sz
         L.yamoe_experts_backward_workspace_bytes.argtypes = [pp]
         L.yamoe_experts_backward.argtypes = [pp] + [vp] * 15 + [sz, vp]
+        L.yamoe_router_topk.argtypes = [vp, vp, vp, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp]
         _lib = L
     return _lib
 
@@ -157,6 +158,21 @@ def down(act, down_proj, down_proj_bias, sched):
     _check(lib().yamoe_down(_p(act), _p(down_proj), _p(down_proj_bias), _p(y), _p(sched), N, E, H, I, dtype_code(act),
                             _stream()), "yamoe_down")
     return y
+
+
+def router_topk(hidden, weight, bias, top_k):
+    """yamoe_router_topk with every optional output: (router_indices int64 [T,K], router_scores [T,E],
+    topk_weights [T,K], logits [T,E])."""
+    _need_gpu(hidden, weight)
+    T, H = hidden.shape
+    E = weight.shape[0]
+    idx = torch.empty(T, top_k, dtype=torch.int64, device=hidden.device)
+    scores = torch.empty(T, E, dtype=hidden.dtype, device=hidden.device)
+    topw = torch.empty(T, top_k, dtype=hidden.dtype, device=hidden.device)
+    logits = torch.empty(T, E, dtype=hidden.dtype, device=hidden.device)
+    _check(lib().yamoe_router_topk(_p(hidden), _p(weight), _p(bias), T, H, E, top_k, dtype_code(hidden), _p(idx), _p(scores),
+                                   _p(topw), _p(logits), _stream()), "yamoe_router_topk")
+    return idx, scores, topw, logits
 
 
 def problem(hidden, router_indices, routing_weights, gate_up_proj, capacity):

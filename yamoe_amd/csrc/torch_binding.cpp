@@ -272,9 +272,38 @@ at::Tensor batch_mm_op(at::Tensor x, at::Tensor weights, at::Tensor batch_sizes,
   return output;
 }
 
+// ---- router step (torch-ext/yamoe/layers.py:128-152): not an op of the reference, which runs it as four torch calls ----
+std::tuple<at::Tensor, at::Tensor> router_topk_op(const at::Tensor &hidden, const at::Tensor &weight,
+                                                  const c10::optional<at::Tensor> &bias, int64_t top_k) {
+  TORCH_CHECK(hidden.is_cuda() && weight.is_cuda(), "router_topk: GPU tensors only");
+  TORCH_CHECK(hidden.dim() == 2 && weight.dim() == 2 && hidden.size(1) == weight.size(1),
+              "router_topk: hidden [T, H] and weight [E, H] expected");
+  TORCH_CHECK(hidden.scalar_type() == at::kBFloat16 || hidden.scalar_type() == at::kHalf,
+              "router_topk: bf16 or fp16 activations only");
+  TORCH_CHECK(weight.scalar_type() == hidden.scalar_type(), "router_topk: weight dtype must match hidden");
+  const int64_t T = hidden.size(0), H = hidden.size(1), E = weight.size(0);
+  at::Tensor x = hidden.contiguous(), w = weight.contiguous(), b;
+  const void *bp = nullptr;
+  if (bias.has_value() && bias->defined()) {
+    TORCH_CHECK(bias->is_cuda() && bias->numel() == E && bias->scalar_type() == hidden.scalar_type(),
+                "router_topk: bias must be [E] of the activation dtype");
+    b = bias->contiguous();
+    bp = b.data_ptr();
+  }
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(hidden.device());
+  at::Tensor indices = at::empty({T, top_k}, hidden.options().dtype(at::kLong));
+  at::Tensor scores = at::empty({T, E}, hidden.options());
+  check_rc(yamoe_router_topk(x.data_ptr(), w.data_ptr(), bp, (int)T, (int)H, (int)E, (int)top_k, dtype_code(hidden, "hidden"),
+                             indices.data_ptr<int64_t>(), scores.data_ptr(), nullptr, nullptr, current_stream()),
+           "yamoe_router_topk");
+  return std::make_tuple(indices, scores);
+}
+
 }  // namespace
 
 TORCH_LIBRARY(_yamoe_amd_ops, ops) {
+  ops.def("router_topk(Tensor hidden, Tensor weight, Tensor? bias, int top_k) -> (Tensor, Tensor)");
+  ops.impl("router_topk", c10::DispatchKey::CUDA, &router_topk_op);
   ops.def("gather(Tensor x, Tensor indices, Tensor bins, Tensor! output, int E, int C, int top_k) -> ()");
   ops.impl("gather", c10::DispatchKey::CUDA, &gather_op);
   ops.def("scatter(Tensor src, Tensor indices, Tensor bins, Tensor weights, Tensor! y, int T, int E, int C, "

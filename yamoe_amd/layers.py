@@ -38,6 +38,12 @@ def experts_autograd(hidden_flat, router_indices, routing_weights, gate_up_proj,
                             down_proj_bias, expert_capacity, num_experts, top_k, enable_router_grads)
 
 
+def router_kernel_takes(x_flat, weight, top_k):
+    """Shapes and dtypes of the fused router kernel (yamoe_router_topk)."""
+    return (x_flat.is_cuda and x_flat.dtype in (torch.bfloat16, torch.float16) and weight.dtype == x_flat.dtype
+            and x_flat.shape[1] % 16 == 0 and weight.shape[0] <= 256 and top_k <= min(16, weight.shape[0]))
+
+
 class Yamoe(torch.nn.Module):
     """Drop-in `forward` for a GPT-OSS MLP block (router + experts), the role of `Yamoe.forward` in
     drbh/yamoe (torch-ext/yamoe/layers.py:106-218).  The host module provides `self.router`
@@ -53,15 +59,22 @@ class Yamoe(torch.nn.Module):
         num_experts = getattr(self, "num_experts", 32)
         top_k = getattr(self, "top_k", 4)
         x_flat = hidden_states.reshape(-1, hidden)
-        logits = torch.nn.functional.linear(x_flat, self.router.weight, self.router.bias)
-        top_vals, router_indices = torch.topk(logits, top_k, dim=-1)
-        top_w = torch.nn.functional.softmax(top_vals, dim=-1, dtype=top_vals.dtype)
-        router_scores = torch.zeros_like(logits).scatter_(1, router_indices, top_w)
+        want_router_grads = torch.is_grad_enabled() and getattr(self, "enable_router_grads", False)
+        if router_kernel_takes(x_flat, self.router.weight, top_k) and not want_router_grads:
+            # linear + top-k + softmax + dense scatter in one kernel
+            router_indices, router_scores = ops.router_topk(x_flat, self.router.weight, self.router.bias, top_k)
+        else:
+            # the same four steps as torch ops on the GPU (fp32 activations, shapes the kernel does not take, or a
+            # router that is being trained: autograd needs the chain)
+            logits = torch.nn.functional.linear(x_flat, self.router.weight, self.router.bias)
+            top_vals, router_indices = torch.topk(logits, top_k, dim=-1)
+            top_w = torch.nn.functional.softmax(top_vals, dim=-1, dtype=top_vals.dtype)
+            router_scores = torch.zeros_like(logits).scatter_(1, router_indices, top_w)
         I = self.experts.down_proj.shape[1]
         gate_up = self.experts.gate_up_proj[:, :, : 2 * I].contiguous()
         gate_up_bias = self.experts.gate_up_proj_bias[:, : 2 * I].contiguous()
         capacity = x_flat.shape[0]
-        if torch.is_grad_enabled() and getattr(self, "enable_router_grads", False):
+        if want_router_grads:
             out = experts_autograd(x_flat, router_indices, router_scores, gate_up, gate_up_bias,
                                    self.experts.down_proj, self.experts.down_proj_bias, capacity, num_experts, top_k,
                                    True)
