@@ -219,7 +219,10 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
   if (n_slabs > 1) issue_b(1);
   if (n_slabs > 2) { issue_b(2); issue_a(1); }
   if (n_slabs > 3) issue_b(3);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // Only slab 0 (the first 12 copies) has to be there to start; the waits of the slab steps below bound the
+  // number of younger copies in flight, and that bound holds for what is left of these 32 as well.
+  if (n_slabs >= 8) asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   read_frags(0, 0, fa0, fb0);
 
@@ -286,8 +289,8 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
   };
   if (n_slabs >= 8) {
     // copies of the (first, second) k-step: A half, B half; whether slab s+1 is read; the vmcnt bound (-1: no wait)
-    slab_step(0, StepCfg<false, false, false, true, true, -1>());
-    slab_step(1, StepCfg<false, true, true, true, true, -1>());
+    slab_step(0, StepCfg<false, false, false, true, true, 16>());
+    slab_step(1, StepCfg<false, true, true, true, true, 6>());
     int s = 2;
     for (; s + 7 < n_slabs; s += 2) {  // steady state
       slab_step(s, StepCfg<true, true, false, true, true, 16>());
@@ -634,10 +637,12 @@ __device__ inline void run_wgrad_tile(const WgradArgs &args, const int tid, cons
 #pragma unroll
         for (int i = 0; i < 4; ++i) { copy_a(s, i); copy_b(s, i); }
       }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // with 8 slabs or more the first four are whole and slab 0 (the first 8 copies) is enough to start with
+    if (n_slabs >= 8) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
     for (int s = 0; s < 4; ++s)
-      if (s < n_slabs && (s + 1) * kBK > rows) zero_tail(s);
+      if (n_slabs < 8 && s < n_slabs && (s + 1) * kBK > rows) zero_tail(s);
     __syncthreads();
     read_frags(0, 0, fa0, fb0);
   }
@@ -682,7 +687,7 @@ __device__ inline void run_wgrad_tile(const WgradArgs &args, const int tid, cons
     }
   };
   if (n_slabs >= 8) {
-    slab_step(0, WStepCfg<false, true, true, false, -1>());
+    slab_step(0, WStepCfg<false, true, true, false, 16>());
     int s = 1;
     for (; s + 5 < n_slabs; ++s) slab_step(s, WStepCfg<true, true, true, false, 16>());
     // s = n_slabs - 5: the last copies (second halves of slab n_slabs - 1) go out in the first k-step of slab n_slabs - 4
