@@ -520,10 +520,10 @@ static int launch(const Args &args, int max_row_tiles, hipStream_t stream) {
 
 // ---- weight gradients: dW[e] = L[rows of e]^T * R[rows of e] -----------------------------------------------
 // (csrc/experts_backward.cu:198, 311).  The contraction runs over the expert's kept rows, so both operands are
-// [k][m] / [k][n] in memory: both stay that way in LDS (4 + 4 single-slab buffers of 32 k-rows x 512 bytes)
-// and both are read with the LDS transpose read.  The last slab of an expert is usually partial: the copies
-// of its missing rows read whatever follows in memory (the caller keeps that readable) and the wave that
-// issued them overwrites them with zeros in LDS before anybody reads the slab.
+// [k][m] / [k][n] in memory: both stay that way in LDS (single-slab buffers of 32 k-rows) and both are read with
+// the LDS transpose read.  The last slab of an expert is usually partial: the copies of its missing rows read
+// whatever follows in memory (the caller keeps that readable) and the wave that issued them overwrites them with
+// zeros in LDS before anybody reads the slab.
 struct WgradArgs {
   const void *A;  // [N, Md] rows in expert order
   const void *B;  // [N, Nd]
@@ -537,14 +537,23 @@ template <bool P1_, bool P2_, bool NEXT_, bool ZERO_, int VM_> struct WStepCfg {
   static constexpr int VM = VM_;
 };
 
+// 128 x 256 tiles with a three-slab ring (72 KB of LDS, at most 256 registers per lane), so that two workgroups
+// share a CU: an expert's contraction is short (its kept rows), a tile spends a third of its time filling the ring
+// and storing its result, and with a second workgroup on the same SIMDs the matrix pipe works through that.
+constexpr int kSmallBM = 128, kSmallStages = 3;
+constexpr int kSmallAStage = kBK * kSmallBM * 2, kSmallBStage = kBK * kBN * 2;  // 8 KB + 16 KB per slab
+constexpr int kSmallBRing = kSmallStages * kSmallAStage;
+constexpr int kSmallRing = kSmallStages * (kSmallAStage + kSmallBStage);
+constexpr int kSmallStaging = kSmallBM * (kBN * 2 + 16);
+constexpr int kSmallLds = kSmallRing > kSmallStaging ? kSmallRing : kSmallStaging;
+
 template <typename T, int NMI>
-__device__ inline void run_wgrad_tile(const WgradArgs &args, const int tid, const int expert, const int m0, const int n0,
-                                      const int rows_m, const long long first, const int rows) {
+__device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid, const int expert, const int m0,
+                                            const int n0, const int rows_m, const long long first, const int rows) {
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   constexpr int NACC = NMI > 0 ? NMI : 1;
-  constexpr int kStage = 16384, kARing = 0, kBRing2 = 4 * kStage;
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds);
 
@@ -559,49 +568,59 @@ __device__ inline void run_wgrad_tile(const WgradArgs &args, const int tid, cons
   const int n_slabs = (rows + kBK - 1) / kBK;
   const long long lda_bytes = (long long)args.Md * (long long)sizeof(T), ldb_bytes = (long long)args.Nd * (long long)sizeof(T);
 
-  // copies: piece i (0..3) of a slab = k rows 8*wave + 2*i + (lane >> 5); LDS position lane & 31 holds piece
-  // pos ^ ((k & 3) << 2) of the 512-byte row
-  uint32_t a_off[4], b_off[4];
+  // A copies: piece i (0..1) = k rows 4*(2*wave + i) + (lane >> 4) of the slab, 256 bytes each; LDS position lane & 15
+  // holds piece pos ^ ((k & 3) << 2).  B copies as in the large kernel: piece i (0..3) = k rows 8*wave + 2*i + (lane >> 5).
+  uint32_t a_off[2], b_off[4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    int k = 4 * (2 * wave + i) + (lane >> 4);
+    int piece = (lane & 15) ^ ((k & 3) << 2);
+    int ca = m0 + piece * 8;
+    if (ca >= args.Md) ca = m0;
+    a_off[i] = (uint32_t)(k * lda_bytes + (long long)(ca - m0) * (long long)sizeof(T));
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     int k = 8 * wave + 2 * i + (lane >> 5);
     int piece = (lane & 31) ^ ((k & 3) << 2);
-    int ca = m0 + piece * 8, cb = n0 + piece * 8;
-    if (ca >= args.Md) ca = m0;  // columns past the end re-read valid ones; never stored
+    int cb = n0 + piece * 8;
     if (cb >= args.Nd) cb = n0;
-    a_off[i] = (uint32_t)(k * lda_bytes + (long long)(ca - m0) * (long long)sizeof(T));
     b_off[i] = (uint32_t)(k * ldb_bytes + (long long)(cb - n0) * (long long)sizeof(T));
   }
   const char *a_base = (const char *)((const T *)args.A + first * args.Md + m0);
   const char *b_base = (const char *)((const T *)args.B + first * args.Nd + n0);
   auto copy_a = [&](int slab, int i) {
     copy16_to_lds(a_base + (long long)slab * kBK * lda_bytes, a_off[i],
-                  lds0 + kARing + (uint32_t)(slab & 3) * kStage + (uint32_t)(8 * wave + 2 * i) * 512u);
+                  lds0 + (uint32_t)(slab % kSmallStages) * kSmallAStage + (uint32_t)(4 * (2 * wave + i)) * 256u);
   };
   auto copy_b = [&](int slab, int i) {
     copy16_to_lds(b_base + (long long)slab * kBK * ldb_bytes, b_off[i],
-                  lds0 + kBRing2 + (uint32_t)(slab & 3) * kStage + (uint32_t)(8 * wave + 2 * i) * 512u);
+                  lds0 + kSmallBRing + (uint32_t)(slab % kSmallStages) * kSmallBStage + (uint32_t)(8 * wave + 2 * i) * 512u);
   };
-  // rows of slab `slab` at or past the end of the expert become zeros (this wave's own pieces, which have landed)
+  auto copy_slab = [&](int slab) {
+    copy_a(slab, 0); copy_b(slab, 0); copy_b(slab, 1); copy_a(slab, 1); copy_b(slab, 2); copy_b(slab, 3);
+  };
   auto zero_tail = [&](int slab) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      int k = 4 * (2 * wave + i) + (lane >> 4);
+      if (slab * kBK + k >= rows)
+        *(u32x4 *)(lds + (slab % kSmallStages) * kSmallAStage + 4 * (2 * wave + i) * 256 + lane * 16) = (u32x4){0, 0, 0, 0};
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       int k = 8 * wave + 2 * i + (lane >> 5);
-      if (slab * kBK + k >= rows) {
-        const int o = (slab & 3) * kStage + (8 * wave + 2 * i) * 512 + lane * 16;
-        *(u32x4 *)(lds + kARing + o) = (u32x4){0, 0, 0, 0};
-        *(u32x4 *)(lds + kBRing2 + o) = (u32x4){0, 0, 0, 0};
-      }
+      if (slab * kBK + k >= rows)
+        *(u32x4 *)(lds + kSmallBRing + (slab % kSmallStages) * kSmallBStage + (8 * wave + 2 * i) * 512 + lane * 16) = (u32x4){0, 0, 0, 0};
     }
   };
 
-  // operand reads: k = ks*16 + g*8 + h*4 + j, 4 columns at c + 16*((lane>>4)&1) + 4*q with j = (lane&15)>>2, q = lane&3
   const int g = lane >> 5, rl = lane & 31, j4 = (lane & 15) >> 2, q4 = lane & 3;
   int a_rd[NACC], b_rd[4];
 #pragma unroll
   for (int mi = 0; mi < NACC; ++mi) {
     int col = (mi * 2 + wm) * 32 + 16 * ((lane >> 4) & 1) + 4 * q4;
-    a_rd[mi] = (g * 8 + j4) * 512 + ((((col >> 3) ^ (j4 << 2))) << 4) + (col & 7) * 2;
+    a_rd[mi] = (g * 8 + j4) * 256 + ((((col >> 3) ^ (j4 << 2))) << 4) + (col & 7) * 2;
   }
 #pragma unroll
   for (int ni = 0; ni < 4; ++ni) {
@@ -610,13 +629,14 @@ __device__ inline void run_wgrad_tile(const WgradArgs &args, const int tid, cons
   }
   u32x4 fa0[NACC], fa1[NACC], fb0[4], fb1[4];
   constexpr int kFrags = NMI > 0 ? 4 + NMI : 0;
-  // fragment order B0, A0, B1, B2, B3, A1, A2, A3
+  // fragment order B0, A0, B1, B2, B3, A1
   auto read_frag = [&](int s, int ks, int f, u32x4 (&fa)[NACC], u32x4 (&fb)[4]) {
     const bool is_a = f == 1 || f >= 5;
     const int idx = is_a ? (f == 1 ? 0 : f - 4) : (f == 0 ? 0 : f - 1);
-    const char *sp = lds + (is_a ? kARing : kBRing2) + (s & 3) * kStage + (is_a ? a_rd[idx] : b_rd[idx]) + ks * 8192;
+    const char *sp = is_a ? lds + (s % kSmallStages) * kSmallAStage + a_rd[idx] + ks * 4096
+                          : lds + kSmallBRing + (s % kSmallStages) * kSmallBStage + b_rd[idx] + ks * 8192;
     u32x2 lo = lds_read_tr16(sp);
-    u32x2 hi = lds_read_tr16(sp + 2048);
+    u32x2 hi = lds_read_tr16(sp + (is_a ? 1024 : 2048));
     u32x4 v = (u32x4){lo[0], lo[1], hi[0], hi[1]};
     if (is_a) fa[idx] = v; else fb[idx] = v;
   };
@@ -625,24 +645,20 @@ __device__ inline void run_wgrad_tile(const WgradArgs &args, const int tid, cons
     for (int f = 0; f < kFrags; ++f) read_frag(s, ks, f, fa, fb);
   };
 
-  // ---- pipeline: as in run_tile, with both operands on single-slab rings ------------------------------------------
-  //   second k-step of slab t: first halves (2 + 2 copies) of slab t + 4;  first k-step of slab t + 1: second halves
-  // i.e. 4 copies per wave in every k-step, and "slab s+1 has landed" means at most 16 younger copies in flight.
+  // pipeline: slab t+3 goes into the buffer slab t leaves at its mid-slab barrier: first half of its copies
+  // (A piece 0, B pieces 0-1) in the second k-step of slab t, second half in the first k-step of slab t+1; "slab
+  // s+1 has landed" = at most 6 younger copies in flight
   constexpr int kMma = 4 * NMI;
   constexpr int kSlots = kMma > 2 ? kMma - 2 : 1;
   if (n_slabs > 0) {
 #pragma unroll
-    for (int s = 0; s < 4; ++s)
-      if (s < n_slabs) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) { copy_a(s, i); copy_b(s, i); }
-      }
-    // with 8 slabs or more the first four are whole and slab 0 (the first 8 copies) is enough to start with
-    if (n_slabs >= 8) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+    for (int s = 0; s < kSmallStages; ++s)
+      if (s < n_slabs) copy_slab(s);
+    if (n_slabs >= 6) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");  // slab 0 is enough to start with
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
-    for (int s = 0; s < 4; ++s)
-      if (n_slabs < 8 && s < n_slabs && (s + 1) * kBK > rows) zero_tail(s);
+    for (int s = 0; s < kSmallStages; ++s)
+      if (n_slabs < 6 && s < n_slabs && (s + 1) * kBK > rows) zero_tail(s);
     __syncthreads();
     read_frags(0, 0, fa0, fb0);
   }
@@ -650,35 +666,34 @@ __device__ inline void run_wgrad_tile(const WgradArgs &args, const int tid, cons
     typedef decltype(cfg) C;
     __builtin_amdgcn_sched_barrier(0);
     {
-      constexpr int kC = C::P1 ? 4 : 0, kItems = kC + kFrags;
+      constexpr int kC = C::P1 ? 3 : 0, kItems = kC + kFrags;
 #pragma unroll
       for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
         if (j < kMma) Mma<T>::run(fa0[j >> 2], fb0[j & 3], acc[j >> 2][j & 3]);
         if (j < kSlots) {
 #pragma unroll
           for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
-            if (i < kC) { if (i < 2) copy_a(s + 3, 2 + i); else copy_b(s + 3, i); }
+            if (i < kC) { if (i == 0) copy_a(s + 2, 1); else copy_b(s + 2, 1 + i); }
             else read_frag(s, 1, i - kC, fa1, fb1);
           }
         }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    if constexpr (C::VM == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-    else if constexpr (C::VM == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    if constexpr (C::VM == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
     else if constexpr (C::VM == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     if constexpr (C::ZERO) zero_tail(s + 1);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
     {
-      constexpr int kC = C::P2 ? 4 : 0, kItems = kC + (C::NEXT ? kFrags : 0);
+      constexpr int kC = C::P2 ? 3 : 0, kItems = kC + (C::NEXT ? kFrags : 0);
 #pragma unroll
       for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
         if (j < kMma) Mma<T>::run(fa1[j >> 2], fb1[j & 3], acc[j >> 2][j & 3]);
         if (j < kSlots) {
 #pragma unroll
           for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
-            if (i < kC) { if (i < 2) copy_a(s + 4, i); else copy_b(s + 4, i - 2); }
+            if (i < kC) { if (i == 0) copy_a(s + 3, 0); else copy_b(s + 3, i - 1); }
             else read_frag(s + 1, 0, i - kC, fa0, fb0);
           }
         }
@@ -686,16 +701,14 @@ __device__ inline void run_wgrad_tile(const WgradArgs &args, const int tid, cons
       }
     }
   };
-  if (n_slabs >= 8) {
-    slab_step(0, WStepCfg<false, true, true, false, 16>());
+  if (n_slabs >= 6) {
+    slab_step(0, WStepCfg<false, true, true, false, 6>());
     int s = 1;
-    for (; s + 5 < n_slabs; ++s) slab_step(s, WStepCfg<true, true, true, false, 16>());
-    // s = n_slabs - 5: the last copies (second halves of slab n_slabs - 1) go out in the first k-step of slab n_slabs - 4
-    slab_step(s, WStepCfg<true, true, true, false, 16>());
-    slab_step(s + 1, WStepCfg<true, false, true, false, 16>());
-    slab_step(s + 2, WStepCfg<false, false, true, false, 8>());
-    slab_step(s + 3, WStepCfg<false, false, true, true, 0>());
-    slab_step(s + 4, WStepCfg<false, false, false, false, -1>());
+    for (; s + 3 < n_slabs; ++s) slab_step(s, WStepCfg<true, true, true, false, 6>());
+    // s = n_slabs - 3
+    slab_step(s, WStepCfg<true, false, true, false, 6>());
+    slab_step(s + 1, WStepCfg<false, false, true, true, 0>());
+    slab_step(s + 2, WStepCfg<false, false, false, false, -1>());
   } else {
     for (int s = 0; s < n_slabs; ++s) {
       if (kFrags > 0) read_frags(s, 1, fa1, fb1);
@@ -704,32 +717,26 @@ __device__ inline void run_wgrad_tile(const WgradArgs &args, const int tid, cons
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       if (s + 1 < n_slabs && (s + 2) * kBK > rows) zero_tail(s + 1);
       __syncthreads();
-      if (s + 4 < n_slabs) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) { copy_a(s + 4, i); copy_b(s + 4, i); }
-      }
+      if (s + kSmallStages < n_slabs) copy_slab(s + kSmallStages);
       if (s + 1 < n_slabs) read_frags(s + 1, 0, fa0, fb0);
 #pragma unroll
       for (int j = 0; j < kMma; ++j) Mma<T>::run(fa1[j >> 2], fb1[j & 3], acc[j >> 2][j & 3]);
     }
   }
 
-  // ---- epilogue: stage the tile in LDS, store whole row segments ------------------------------------------------
+  // epilogue: stage the tile in LDS, store whole row segments
   constexpr int stride = kBN * 2 + 16;
   const int rsub = g * 4;
   __syncthreads();
   {
     char *lp0 = lds + (wm * 32 + rsub) * stride + (wn * 128 + rl) * 2;
-    char *lp1 = lp0 + 128 * stride;
 #pragma unroll
     for (int ni = 0; ni < 4; ++ni)
 #pragma unroll
       for (int mi = 0; mi < NMI; ++mi)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          char *q = (mi < 2 ? lp0 : lp1) + ((mi & 1) * 64 + 8 * (v >> 2) + (v & 3)) * stride + ni * 64;
-          *(T *)q = ElemTraits<T>::from_f32(acc[mi][ni][v]);
-        }
+        for (int v = 0; v < 16; ++v)
+          *(T *)(lp0 + (mi * 64 + 8 * (v >> 2) + (v & 3)) * stride + ni * 64) = ElemTraits<T>::from_f32(acc[mi][ni][v]);
   }
   __syncthreads();
   {
@@ -744,10 +751,8 @@ __device__ inline void run_wgrad_tile(const WgradArgs &args, const int tid, cons
 }
 
 template <typename T>
-__global__ __launch_bounds__(kThreads) void wgrad_async_kernel(const WgradArgs args) {
+__global__ __launch_bounds__(kThreads, 2) void wgrad_small_kernel(const WgradArgs args) {
   const int tid = threadIdx.x, wave = tid >> 6, wm = wave >> 1;
-  // tile list: expert, then column tile, then row tiles; workgroup b runs on XCD b % 8, which takes a contiguous
-  // eighth of the list
   const int per_expert = args.n_m_tiles * args.n_n_tiles;
   const int total = args.E * per_expert;
   const int total8 = (total + kXcds - 1) / kXcds * kXcds;
@@ -756,19 +761,17 @@ __global__ __launch_bounds__(kThreads) void wgrad_async_kernel(const WgradArgs a
   const int L = (b % kXcds) * (total8 / kXcds) + b / kXcds;
   if (L >= total) return;
   const int expert = L / per_expert, r = L - expert * per_expert;
-  const int n0 = (r / args.n_m_tiles) * kBN, m0 = (r % args.n_m_tiles) * kBM;
-  const int rows_m = min(kBM, args.Md - m0);
+  const int n0 = (r / args.n_m_tiles) * kBN, m0 = (r % args.n_m_tiles) * kSmallBM;
+  const int rows_m = min(kSmallBM, args.Md - m0);
   int rows = min(args.counts[expert], args.capacity);
   if (rows < 0) rows = 0;
   const long long first = args.offsets[expert];
   const int n_blocks32 = (rows_m + 31) >> 5;
   const int n_mi = (n_blocks32 - wm + 1) >> 1;
   switch (n_mi) {
-    case 4: run_wgrad_tile<T, 4>(args, tid, expert, m0, n0, rows_m, first, rows); break;
-    case 3: run_wgrad_tile<T, 3>(args, tid, expert, m0, n0, rows_m, first, rows); break;
-    case 2: run_wgrad_tile<T, 2>(args, tid, expert, m0, n0, rows_m, first, rows); break;
-    case 1: run_wgrad_tile<T, 1>(args, tid, expert, m0, n0, rows_m, first, rows); break;
-    default: run_wgrad_tile<T, 0>(args, tid, expert, m0, n0, rows_m, first, rows); break;
+    case 2: run_wgrad_tile_small<T, 2>(args, tid, expert, m0, n0, rows_m, first, rows); break;
+    case 1: run_wgrad_tile_small<T, 1>(args, tid, expert, m0, n0, rows_m, first, rows); break;
+    default: run_wgrad_tile_small<T, 0>(args, tid, expert, m0, n0, rows_m, first, rows); break;
   }
 }
 
@@ -826,14 +829,14 @@ int gemm_async_wgrad(const void *L, const void *R, void *dW, const int *counts, 
   async::WgradArgs a = {};
   a.A = L; a.B = R; a.C = dW; a.counts = counts; a.offsets = offsets; a.capacity = capacity;
   a.E = E; a.Md = Md; a.Nd = Nd;
-  a.n_m_tiles = ceil_div(Md, async::kBM);
+  a.n_m_tiles = ceil_div(Md, async::kSmallBM);
   a.n_n_tiles = ceil_div(Nd, async::kBN);
-  auto kernel = async::wgrad_async_kernel<T>;
+  auto kernel = async::wgrad_small_kernel<T>;
   static bool attr_done = false;  // benign race: the attribute call is idempotent
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, async::kLds);
+    hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, async::kSmallLds);
     if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(MaxDynamicSharedMemorySize=%d): %s", async::kLds, hipGetErrorString(e));
+      set_error("hipFuncSetAttribute(MaxDynamicSharedMemorySize=%d): %s", async::kSmallLds, hipGetErrorString(e));
       return (int)e;
     }
     attr_done = true;
@@ -841,8 +844,8 @@ int gemm_async_wgrad(const void *L, const void *R, void *dW, const int *counts, 
   long long total = (long long)E * a.n_m_tiles * a.n_n_tiles;
   if (total <= 0) return 0;
   total = (total + kXcds - 1) / kXcds * kXcds;
-  hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(async::kThreads), async::kLds, stream, a);
-  return check_launch("wgrad_async_kernel");
+  hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(async::kThreads), async::kSmallLds, stream, a);
+  return check_launch("wgrad_small_kernel");
 }
 
 #define YAMOE_INSTANTIATE_ASYNC(T)                                                                               \
