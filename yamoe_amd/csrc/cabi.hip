@@ -32,8 +32,8 @@ template <typename T>
 int launch_combine(const void *, const int *, const void *, int, const void *, int, void *, int, int, int, int,
                    hipStream_t);
 template <typename T>
-int launch_combine_backward(const void *, const void *, const int *, const int *, const void *, int, const void *,
-                            int, void *, void *, int, int, int, int, hipStream_t);
+int launch_combine_backward(const void *, const void *, const int *, const int *, const void *, int, const void *, int,
+                            void *, float *, float *, int, int, int, int, hipStream_t);
 template <typename T>
 int launch_expert_colsum(const void *, const int *, const int *, int, void *, int, int, hipStream_t);
 template <typename T>
@@ -42,10 +42,12 @@ int gemm_gate_up(const void *, const int *, const void *, const void *, void *, 
 template <typename T>
 int gemm_down(const void *, const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);
 template <typename T>
-int gemm_dgrad(const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);
+int gemm_dgrad(const void *, const int *, int, const void *, void *, const void *, int, int, int, int, hipStream_t);
 template <typename T>
 int gemm_wgrad(const void *, const void *, void *, const int *, const int *, int, int, int, int, hipStream_t);
-template <typename T> int glu_backward_rows(const void *, const void *, void *, long long, hipStream_t);
+template <typename T>
+int glu_backward_rows(const void *, const void *, const float *, const float *, const int *, const int *, const void *,
+                      int, int, void *, void *, int, int, int, int, hipStream_t);
 template <typename T>
 int stream_gate_up(const void *, const int *, const void *, const void *, void *, void *, const void *, int, int, int,
                    int, int, hipStream_t);
@@ -58,7 +60,8 @@ int gemm_async_gate_up(const void *, const int *, const void *, const void *, vo
 template <typename T>
 int gemm_async_down(const void *, const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);
 template <typename T>
-int gemm_async_dgrad(const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);
+int gemm_async_dgrad(const void *, const int *, int, const void *, void *, const void *, int, int, int, int,
+                     hipStream_t);
 template <typename T>
 int gemm_async_wgrad(const void *, const void *, void *, const int *, const int *, int, int, int, int, hipStream_t);
 bool gemm_async_supported(int Kd, int Nd, int lda, int ldb, long long a_span_bytes);
@@ -87,13 +90,16 @@ static int tiles_down(const void *act, const void *w, const void *bias, void *y,
   return gemm_down<T>(act, w, bias, y, sched, N, E, H, I, stream);
 }
 
+// g_rows == nullptr: g holds one row per sorted row; otherwise row p of the product reads g[g_rows[p] / g_div]
+// (g_span_bytes = size of the gathered tensor)
 template <typename T>
-static int tiles_dgrad(const void *g, const void *w, void *out, const void *sched, int N, int E, int Kd, int Nd,
-                       hipStream_t stream) {
+static int tiles_dgrad(const void *g, const int *g_rows, int g_div, long long g_span_bytes, const void *w, void *out,
+                       const void *sched, int N, int E, int Kd, int Nd, hipStream_t stream) {
   if constexpr (sizeof(T) == 2) {
-    if (gemm_async_supported(Kd, Nd, Kd, Kd, 0)) return gemm_async_dgrad<T>(g, w, out, sched, N, E, Kd, Nd, stream);
+    if (gemm_async_supported(Kd, Nd, Kd, Kd, g_rows ? g_span_bytes : 0))
+      return gemm_async_dgrad<T>(g, g_rows, g_div, w, out, sched, N, E, Kd, Nd, stream);
   }
-  return gemm_dgrad<T>(g, w, out, sched, N, E, Kd, Nd, stream);
+  return gemm_dgrad<T>(g, g_rows, g_div, w, out, sched, N, E, Kd, Nd, stream);
 }
 
 template <typename T>
@@ -184,6 +190,7 @@ static size_t carve_forward(const yamoe_problem *p, void *ws, ForwardBuffers *b)
 struct BackwardBuffers {
   ForwardBuffers f;
   void *x_perm, *pre, *g_y_perm, *d_act, *d_pre, *d_x_perm;
+  float *w_sorted, *dot_bias;
 };
 
 static size_t carve_backward(const yamoe_problem *p, void *ws, BackwardBuffers *b) {
@@ -197,6 +204,8 @@ static size_t carve_backward(const yamoe_problem *p, void *ws, BackwardBuffers *
   // d_act [N, I] reuses the y_perm region (dead after the combine backward)
   b->d_act = b->f.y_perm;
   b->d_x_perm = c.take(N * p->H * es);
+  b->w_sorted = (float *)c.take(N * sizeof(float));
+  b->dot_bias = (float *)c.take(N * sizeof(float));
   // the weight-gradient kernel's copies of an expert's last, partial slab of rows run up to 32 rows past the
   // end of its operand buffers; every operand is followed by another buffer of this workspace, and this pad
   // covers the case where those are smaller than 32 rows of the widest operand
@@ -255,22 +264,24 @@ static int backward_impl(const yamoe_problem *p, const void *gy, const void *x, 
   YAMOE_TRY(yamoe_route(idx, p->idx_i64, N, E, cap, b.f.sorted_expert, b.f.sorted_idx, b.f.counts, b.f.offsets,
                         b.f.inv_pos, b.f.route_ws, b.f.route_ws_bytes, st));
   YAMOE_TRY(yamoe_build_schedule(b.f.counts, b.f.offsets, N, E, cap, 0, b.f.schedule, b.f.schedule_bytes, st));
-  // forward recompute, keeping the pre-activations
+  // forward recompute of the first product only: activations and pre-activations
   YAMOE_TRY(launch_permute<T>(x, b.f.sorted_idx, b.x_perm, N, p->K, H, stream));
   YAMOE_TRY(tiles_gate_up<T>(x, b.f.sorted_idx, wgu, bgu, b.f.act, b.pre, b.f.schedule, N, p->K, E, H, I, stream));
-  YAMOE_TRY(tiles_down<T>(b.f.act, wd, bd, b.f.y_perm, b.f.schedule, N, E, H, I, stream));
-  // combine backward: g_y_perm = grad_out[tok] * w, d_routing = <grad_out[tok], y_perm>
-  YAMOE_TRY(launch_combine_backward<T>(gy, b.f.y_perm, b.f.sorted_idx, b.f.inv_pos, idx, p->idx_i64, rw, p->rw_cols,
-                                       b.g_y_perm, d_rw, N, p->K, E, H, stream));
-  // down projection
+  // combine backward: g_y_perm = grad_out[tok] * w, and the bias part of the routing gradient
+  YAMOE_TRY(launch_combine_backward<T>(gy, bd, b.f.sorted_idx, b.f.inv_pos, idx, p->idx_i64, rw, p->rw_cols, b.g_y_perm,
+                                       b.w_sorted, b.dot_bias, N, p->K, E, H, stream));
+  // down projection: bias and weight gradients from the weighted rows; the input gradient from the un-weighted
+  // rows of grad_out, gathered by token (its dot with the activations is the rest of the routing gradient)
   YAMOE_TRY(launch_expert_colsum<T>(b.g_y_perm, b.f.counts, b.f.offsets, cap, d_bd, E, H, stream));
-  YAMOE_TRY(tiles_dgrad<T>(b.g_y_perm, wd, b.d_act, b.f.schedule, N, E, /*Kd=*/H, /*Nd=*/I, stream));
+  YAMOE_TRY(tiles_dgrad<T>(gy, b.f.sorted_idx, p->K, (long long)p->T * H * (long long)es, wd, b.d_act, b.f.schedule, N, E,
+                           /*Kd=*/H, /*Nd=*/I, stream));
   YAMOE_TRY(tiles_wgrad<T>(b.f.act, b.g_y_perm, d_wd, b.f.counts, b.f.offsets, cap, E, /*Md=*/I, /*Nd=*/H, stream));
-  // GLU
-  YAMOE_TRY(glu_backward_rows<T>(b.d_act, b.pre, b.d_pre, (long long)N * I, stream));
+  // GLU backward (scaled by the routing weight) and the routing gradient
+  YAMOE_TRY(glu_backward_rows<T>(b.d_act, b.pre, b.w_sorted, b.dot_bias, b.f.sorted_idx, b.f.inv_pos, idx, p->idx_i64,
+                                 p->rw_cols, b.d_pre, d_rw, N, p->K, E, I, stream));
   // gate_up projection
   YAMOE_TRY(launch_expert_colsum<T>(b.d_pre, b.f.counts, b.f.offsets, cap, d_bgu, E, 2 * I, stream));
-  YAMOE_TRY(tiles_dgrad<T>(b.d_pre, wgu, b.d_x_perm, b.f.schedule, N, E, /*Kd=*/2 * I, /*Nd=*/H, stream));
+  YAMOE_TRY(tiles_dgrad<T>(b.d_pre, nullptr, 1, 0, wgu, b.d_x_perm, b.f.schedule, N, E, /*Kd=*/2 * I, /*Nd=*/H, stream));
   YAMOE_TRY(tiles_wgrad<T>(b.x_perm, b.d_pre, d_wgu, b.f.counts, b.f.offsets, cap, E, /*Md=*/H, /*Nd=*/2 * I, stream));
   // permute backward: d_hidden[t] = sum_k d_x_perm[inv_pos[t,k]]
   YAMOE_TRY(launch_combine<T>(b.d_x_perm, b.f.inv_pos, idx, p->idx_i64, nullptr, p->K, d_x, p->T, p->K, E, H, stream));

@@ -485,23 +485,6 @@ __global__ __launch_bounds__(kGemmThreads) void grouped_gemm_kernel(const GemmAr
   }
 }
 
-// GLU backward on rows: d_act [rows, I] and the stored pre-activations [rows, 2I] give the
-// interleaved (gate, up) pre-activation gradients [rows, 2I] (csrc/experts_backward.cu:285-305).
-template <typename T>
-__global__ __launch_bounds__(256) void glu_backward_rows_kernel(const T *__restrict__ d_act,
-                                                                const T *__restrict__ pre,
-                                                                T *__restrict__ d_pre, long long n_pairs) {
-  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  long long stride = (long long)gridDim.x * blockDim.x;
-  for (; i < n_pairs; i += stride) {
-    float G = ElemTraits<T>::to_f32(pre[2 * i]), U = ElemTraits<T>::to_f32(pre[2 * i + 1]);
-    float dG, dU;
-    glu_backward(G, U, ElemTraits<T>::to_f32(d_act[i]), dG, dU);
-    d_pre[2 * i] = ElemTraits<T>::from_f32(dG);
-    d_pre[2 * i + 1] = ElemTraits<T>::from_f32(dU);
-  }
-}
-
 // Experts that own no kept rows need no special case in the weight-gradient product: k_len = 0
 // leaves the accumulators at zero and the epilogue stores them.
 
@@ -549,16 +532,20 @@ int gemm_down(const void *act, const void *w, const void *bias, void *y, const v
   return launch_gemm<T, OP_KCONTIG, OP_TRANSPOSED, EPI_STORE, PROB_ROWS, false>(a, sched_max_row_tiles(N, E), stream);
 }
 
-// d_out[p,:] = g[p,:] . W[e]^T with W[e] = [n_out, k] row-major, i.e. k-contiguous "B rows".
+// d_out[p,:] = g[p,:] . W[e]^T with W[e] = [n_out, k] row-major, i.e. k-contiguous "B rows".  With g_rows the
+// source row of p is g_rows[p] / g_div (rows of a [T, Kd] tensor gathered by token).
 template <typename T>
-int gemm_dgrad(const void *g, const void *w, void *d_out, const void *sched, int N, int E, int Kd, int Nd,
-               hipStream_t stream) {
+int gemm_dgrad(const void *g, const int *g_rows, int g_div, const void *w, void *d_out, const void *sched, int N, int E,
+               int Kd, int Nd, hipStream_t stream) {
   GemmArgs a = {};
   a.A = g; a.B = w; a.C = d_out; a.sched = (const int *)sched;
+  a.a_rows = g_rows; a.a_div = g_div;
   a.Kd = Kd; a.Nd = Nd; a.lda = Kd; a.ldb = Kd; a.ldc = Nd;
   a.b_expert_stride = (long long)Nd * Kd;
   a.n_col_tiles = ceil_div(Nd, kBN);
   a.N = N; a.E = E;
+  if (g_rows != nullptr)
+    return launch_gemm<T, OP_KCONTIG, OP_KCONTIG, EPI_STORE, PROB_ROWS, true>(a, sched_max_row_tiles(N, E), stream);
   return launch_gemm<T, OP_KCONTIG, OP_KCONTIG, EPI_STORE, PROB_ROWS, false>(a, sched_max_row_tiles(N, E), stream);
 }
 
@@ -576,25 +563,15 @@ int gemm_wgrad(const void *L, const void *R, void *dW, const int *counts, const 
   return launch_gemm<T, OP_TRANSPOSED, OP_TRANSPOSED, EPI_STORE, PROB_WGRAD, false>(a, E * a.n_row_tiles_wgrad, stream);
 }
 
-template <typename T>
-int glu_backward_rows(const void *d_act, const void *pre, void *d_pre, long long n_pairs, hipStream_t stream) {
-  if (n_pairs == 0) return 0;
-  long long blocks = (n_pairs + 255) / 256;
-  if (blocks > 256 * 32) blocks = 256 * 32;
-  hipLaunchKernelGGL(glu_backward_rows_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, (const T *)d_act,
-                     (const T *)pre, (T *)d_pre, n_pairs);
-  return check_launch("glu_backward_rows_kernel");
-}
-
 #define YAMOE_INSTANTIATE_GEMM(T)                                                                                   \
   template int gemm_gate_up<T>(const void *, const int *, const void *, const void *, void *, void *, const void *, \
                                int, int, int, int, int, hipStream_t);                                               \
   template int gemm_down<T>(const void *, const void *, const void *, void *, const void *, int, int, int, int,     \
                             hipStream_t);                                                                           \
-  template int gemm_dgrad<T>(const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);    \
-  template int gemm_wgrad<T>(const void *, const void *, void *, const int *, const int *, int, int, int, int,      \
+  template int gemm_dgrad<T>(const void *, const int *, int, const void *, void *, const void *, int, int, int, int, \
                              hipStream_t);                                                                          \
-  template int glu_backward_rows<T>(const void *, const void *, void *, long long, hipStream_t);
+  template int gemm_wgrad<T>(const void *, const void *, void *, const int *, const int *, int, int, int, int,      \
+                             hipStream_t);
 YAMOE_INSTANTIATE_GEMM(float)
 YAMOE_INSTANTIATE_GEMM(bf16_t)
 YAMOE_INSTANTIATE_GEMM(f16_t)

@@ -808,14 +808,17 @@ int gemm_async_down(const void *act, const void *w, const void *bias, void *y, c
 
 // C[rows, Nd] = A[rows, Kd] * W[e]^T with W[e] stored [Nd, Kd]: the input gradients of both projections
 // (csrc/experts_backward.cu:279-282, 309-311), without materialising a transposed weight.
+// With g_rows the source row of sorted row p is g_rows[p] / g_div (rows of a [T, Kd] tensor gathered by token).
 template <typename T>
-int gemm_async_dgrad(const void *g, const void *w, void *out, const void *sched, int N, int E, int Kd, int Nd,
-                     hipStream_t stream) {
+int gemm_async_dgrad(const void *g, const int *g_rows, int g_div, const void *w, void *out, const void *sched, int N,
+                     int E, int Kd, int Nd, hipStream_t stream) {
   async::Args a = {};
   a.A = g; a.B = w; a.bias = nullptr; a.C = out; a.sched = (const int *)sched;
+  a.a_rows = g_rows; a.a_div = g_div;
   a.Kd = Kd; a.Nd = Nd; a.lda = Kd; a.ldb = Kd; a.ldc = Nd;
   a.b_expert_stride = (long long)Nd * Kd;
   a.n_col_tiles = ceil_div(Nd, async::kBN);
+  if (g_rows != nullptr) return async::launch<T, async::EPI_STORE, true, true>(a, sched_max_row_tiles(N, E), stream);
   return async::launch<T, async::EPI_STORE, false, true>(a, sched_max_row_tiles(N, E), stream);
 }
 
@@ -853,7 +856,8 @@ int gemm_async_wgrad(const void *L, const void *R, void *dW, const int *counts, 
                                      const void *, int, int, int, int, int, hipStream_t);                        \
   template int gemm_async_down<T>(const void *, const void *, const void *, void *, const void *, int, int, int, \
                                   int, hipStream_t);                                                             \
-  template int gemm_async_dgrad<T>(const void *, const void *, void *, const void *, int, int, int, int, hipStream_t); \
+  template int gemm_async_dgrad<T>(const void *, const int *, int, const void *, void *, const void *, int, int, int,  \
+                                   int, hipStream_t);                                                                  \
   template int gemm_async_wgrad<T>(const void *, const void *, void *, const int *, const int *, int, int, int, int,    \
                                    hipStream_t);
 YAMOE_INSTANTIATE_ASYNC(bf16_t)

@@ -109,16 +109,19 @@ __global__ __launch_bounds__(kRowThreads) void combine_kernel(
   }
 }
 
-// Backward of the combine (csrc/experts_backward.cu:37-89) in sorted-row order:
-//   g_y_perm[p,:] = grad_out[tok,:] * w(tok,slot)          for kept rows p
-//   d_sel[flat]   = <grad_out[tok,:], y_perm[p,:]>         (fp32 wave-parallel dot)
-// and the dense routing gradient d_routing[tok, expert] = d_sel (zero elsewhere is the caller's
-// fill).  Dropped slots get no row and a zero gradient.
+// Backward of the combine (csrc/experts_backward.cu:37-89) in sorted-row order, for kept rows p = (tok, slot):
+//   g_y_perm[p,:] = grad_out[tok,:] * w(tok,slot)
+//   w_sorted[p]   = w(tok,slot)
+//   dot_bias[p]   = <grad_out[tok,:], down_bias[expert,:]>
+// The routing gradient is <grad_out[tok], y[p]> with y[p] = act[p] . W_down + down_bias (the expert's output row
+// before weighting).  Instead of recomputing y, the backward uses <grad_out[tok] . W_down^T, act[p]> + dot_bias[p]:
+// the first factor is the input gradient of the down projection of the un-weighted row, which the backward needs
+// anyway; glu_backward_rows_kernel finishes the sum.  Dropped slots get no row and a zero gradient.
 template <typename T, bool I64>
 __global__ __launch_bounds__(kRowThreads) void combine_backward_kernel(
-    const T *__restrict__ grad_out, const T *__restrict__ y_perm, const int *__restrict__ sorted_idx,
-    const int *__restrict__ inv_pos, const void *__restrict__ idx, const T *__restrict__ rw,
-    int rw_cols, T *__restrict__ g_y_perm, T *__restrict__ d_routing, int N, int K, int E, int H) {
+    const T *__restrict__ grad_out, const T *__restrict__ down_bias, const int *__restrict__ sorted_idx,
+    const int *__restrict__ inv_pos, const void *__restrict__ idx, const T *__restrict__ rw, int rw_cols,
+    T *__restrict__ g_y_perm, float *__restrict__ w_sorted, float *__restrict__ dot_bias, int N, int K, int E, int H) {
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = blockIdx.x * kRowWaves + threadIdx.x / kWave;
   const int n_waves = gridDim.x * kRowWaves;
@@ -127,22 +130,64 @@ __global__ __launch_bounds__(kRowThreads) void combine_backward_kernel(
     if (inv_pos[flat] != p) continue;  // dropped or invalid expert id
     int t = flat / K, k = flat - t * K;
     float w = slot_weight<T, I64>(rw, idx, t, k, K, E, rw_cols);
+    long long e = I64 ? ((const long long *)idx)[flat] : (long long)((const int *)idx)[flat];
     const T *g = grad_out + (size_t)t * H;
-    const T *y = y_perm + (size_t)p * H;
+    const T *bd = down_bias + (size_t)e * H;
     T *o = g_y_perm + (size_t)p * H;
     float dot = 0.0f;
     for (int c = lane; c < H; c += kWave) {
       float gv = ElemTraits<T>::to_f32(g[c]);
-      dot += gv * ElemTraits<T>::to_f32(y[c]);
+      dot += gv * ElemTraits<T>::to_f32(bd[c]);
       o[c] = ElemTraits<T>::from_f32(gv * w);
     }
     for (int d = kWave / 2; d > 0; d >>= 1) dot += __shfl_xor(dot, d);
     if (lane == 0) {
+      w_sorted[p] = w;
+      dot_bias[p] = dot;
+    }
+  }
+}
+
+// GLU backward on kept rows (csrc/experts_backward.cu:285-305) plus the rest of the routing gradient:
+//   d_act[p,:] is the input gradient of the down projection for the UN-weighted output gradient of row p,
+//   d_pre[p,:] = w_sorted[p] * glu'(pre[p,:]) applied to d_act[p,:]      (interleaved gate/up columns)
+//   d_routing[tok, expert] = <d_act[p,:], glu(pre[p,:])> + dot_bias[p]
+// One wave per row; d_routing is written once per kept (token, slot).
+template <typename T, bool I64>
+__global__ __launch_bounds__(kRowThreads) void glu_backward_rows_kernel(
+    const T *__restrict__ d_act, const T *__restrict__ pre, const float *__restrict__ w_sorted,
+    const float *__restrict__ dot_bias, const int *__restrict__ sorted_idx, const int *__restrict__ inv_pos,
+    const void *__restrict__ idx, int rw_cols, T *__restrict__ d_pre, T *__restrict__ d_routing, int N, int K, int E,
+    int I) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = blockIdx.x * kRowWaves + threadIdx.x / kWave;
+  const int n_waves = gridDim.x * kRowWaves;
+  for (int p = wave; p < N; p += n_waves) {
+    int flat = sorted_idx[p];
+    if (inv_pos[flat] != p) continue;
+    const float w = w_sorted[p];
+    const T *da = d_act + (size_t)p * I;
+    const T *pr = pre + (size_t)p * 2 * I;
+    T *dp = d_pre + (size_t)p * 2 * I;
+    float dot = 0.0f;
+    for (int c = lane; c < I; c += kWave) {
+      float G = ElemTraits<T>::to_f32(pr[2 * c]), U = ElemTraits<T>::to_f32(pr[2 * c + 1]);
+      float dh = ElemTraits<T>::to_f32(da[c]);
+      float dG, dU;
+      glu_backward(G, U, dh * w, dG, dU);
+      dot += dh * glu_forward(G, U);
+      dp[2 * c] = ElemTraits<T>::from_f32(dG);
+      dp[2 * c + 1] = ElemTraits<T>::from_f32(dU);
+    }
+    for (int d = kWave / 2; d > 0; d >>= 1) dot += __shfl_xor(dot, d);
+    if (lane == 0) {
+      int t = flat / K, k = flat - t * K;
+      float v = dot + dot_bias[p];
       if (rw_cols == K && rw_cols != E) {
-        d_routing[(size_t)t * K + k] = ElemTraits<T>::from_f32(dot);
+        d_routing[(size_t)t * K + k] = ElemTraits<T>::from_f32(v);
       } else {
         long long e = I64 ? ((const long long *)idx)[flat] : (long long)((const int *)idx)[flat];
-        d_routing[(size_t)t * E + e] = ElemTraits<T>::from_f32(dot);
+        d_routing[(size_t)t * E + e] = ElemTraits<T>::from_f32(v);
       }
     }
   }
@@ -240,21 +285,37 @@ int launch_combine(const void *y_perm, const int *inv_pos, const void *idx, int 
 }
 
 template <typename T>
-int launch_combine_backward(const void *grad_out, const void *y_perm, const int *sorted_idx,
-                            const int *inv_pos, const void *idx, int idx_i64, const void *rw,
-                            int rw_cols, void *g_y_perm, void *d_routing, int N, int K, int E, int H,
-                            hipStream_t stream) {
+int launch_combine_backward(const void *grad_out, const void *down_bias, const int *sorted_idx, const int *inv_pos,
+                            const void *idx, int idx_i64, const void *rw, int rw_cols, void *g_y_perm, float *w_sorted,
+                            float *dot_bias, int N, int K, int E, int H, hipStream_t stream) {
   if (N == 0) return 0;
   int blocks = min(ceil_div(N, kRowWaves), 256 * 16);
   if (idx_i64)
     hipLaunchKernelGGL((combine_backward_kernel<T, true>), dim3(blocks), dim3(kRowThreads), 0, stream,
-                       (const T *)grad_out, (const T *)y_perm, sorted_idx, inv_pos, idx, (const T *)rw,
-                       rw_cols, (T *)g_y_perm, (T *)d_routing, N, K, E, H);
+                       (const T *)grad_out, (const T *)down_bias, sorted_idx, inv_pos, idx, (const T *)rw, rw_cols,
+                       (T *)g_y_perm, w_sorted, dot_bias, N, K, E, H);
   else
     hipLaunchKernelGGL((combine_backward_kernel<T, false>), dim3(blocks), dim3(kRowThreads), 0, stream,
-                       (const T *)grad_out, (const T *)y_perm, sorted_idx, inv_pos, idx, (const T *)rw,
-                       rw_cols, (T *)g_y_perm, (T *)d_routing, N, K, E, H);
+                       (const T *)grad_out, (const T *)down_bias, sorted_idx, inv_pos, idx, (const T *)rw, rw_cols,
+                       (T *)g_y_perm, w_sorted, dot_bias, N, K, E, H);
   return check_launch("combine_backward_kernel");
+}
+
+template <typename T>
+int glu_backward_rows(const void *d_act, const void *pre, const float *w_sorted, const float *dot_bias,
+                      const int *sorted_idx, const int *inv_pos, const void *idx, int idx_i64, int rw_cols, void *d_pre,
+                      void *d_routing, int N, int K, int E, int I, hipStream_t stream) {
+  if (N == 0) return 0;
+  int blocks = min(ceil_div(N, kRowWaves), 256 * 16);
+  if (idx_i64)
+    hipLaunchKernelGGL((glu_backward_rows_kernel<T, true>), dim3(blocks), dim3(kRowThreads), 0, stream, (const T *)d_act,
+                       (const T *)pre, w_sorted, dot_bias, sorted_idx, inv_pos, idx, rw_cols, (T *)d_pre, (T *)d_routing, N,
+                       K, E, I);
+  else
+    hipLaunchKernelGGL((glu_backward_rows_kernel<T, false>), dim3(blocks), dim3(kRowThreads), 0, stream, (const T *)d_act,
+                       (const T *)pre, w_sorted, dot_bias, sorted_idx, inv_pos, idx, rw_cols, (T *)d_pre, (T *)d_routing, N,
+                       K, E, I);
+  return check_launch("glu_backward_rows_kernel");
 }
 
 template <typename T>
@@ -274,9 +335,12 @@ int launch_expert_colsum(const void *src, const int *counts, const int *offsets,
   template int launch_permute<T>(const void *, const int *, void *, int, int, int, hipStream_t);        \
   template int launch_combine<T>(const void *, const int *, const void *, int, const void *, int,       \
                                  void *, int, int, int, int, hipStream_t);                              \
-  template int launch_combine_backward<T>(const void *, const void *, const int *, const int *,        \
-                                          const void *, int, const void *, int, void *, void *, int,   \
-                                          int, int, int, hipStream_t);                                  \
+  template int launch_combine_backward<T>(const void *, const void *, const int *, const int *, const void *,   \
+                                          int, const void *, int, void *, float *, float *, int, int, int, int,  \
+                                          hipStream_t);                                                          \
+  template int glu_backward_rows<T>(const void *, const void *, const float *, const float *, const int *,      \
+                                    const int *, const void *, int, int, void *, void *, int, int, int, int,     \
+                                    hipStream_t);                                                                \
   template int launch_expert_colsum<T>(const void *, const int *, const int *, int, void *, int, int,  \
                                        hipStream_t);
 YAMOE_INSTANTIATE_ROWS(float)
