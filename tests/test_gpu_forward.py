@@ -142,3 +142,14 @@ def test_op_rejects_bad_arguments(gpu):
         yamoe_amd.experts(a[0], a[1], a[2].float(), *a[3:], 8, 4, 2)  # dtype mismatch
     with pytest.raises(RuntimeError):
         yamoe_amd.experts(a[0], a[1].float(), *a[2:], 8, 4, 2)  # indices must be integers
+
+
+def test_sweep_point_runs(gpu):
+    """One small point of the reference's timing sweep (perf_plot.py:29-39 shapes, scaled down) through the sweep
+    driver: fp16, unit-variance weights, both capacity conventions."""
+    from yamoe_amd import sweep
+    r = sweep.run_point(2, 64, 128, 8, 2, iters=2, warmup=1, capacity="tokens")
+    assert r["kept_assignments"] == 2 * 64 * 2 and r["ms"] > 0 and r["finite"]
+    r = sweep.run_point(2, 64, 128, 8, 2, iters=2, warmup=1, capacity="seq")
+    assert r["kept_assignments"] <= 2 * 64 * 2 and r["capacity"] == 64
+    assert len(sweep.CONFIGS) == 6 and sweep.BATCH_SIZES == [1, 2, 4, 8, 16, 32, 64]
