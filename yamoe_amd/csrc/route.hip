@@ -61,7 +61,7 @@ __device__ inline void wave_histogram(const void *idx, int seg_begin, int seg_en
 // the next free sorted position per bucket.
 template <bool I64>
 __device__ inline void wave_place(const void *idx, int seg_begin, int seg_end, int E, int capacity,
-                                  volatile int *cursor, const int *offsets_lds,
+                                  int *cursor, const int *offsets_lds,
                                   int *sorted_expert, int *sorted_idx, int *inv_pos) {
   const int lane = threadIdx.x & (kWave - 1);
   const int key_bits = bits_for(E + 1);
@@ -93,8 +93,10 @@ __device__ inline void wave_place(const void *idx, int seg_begin, int seg_end, i
       inv_pos[i] = kept ? pos : -1;
       if (rank == 0) cursor[key] = start + __popcll(peers);
     }
+    // the cursor is private to this wave and LDS operations of one wave complete in order: the next step's
+    // read sees this step's write without a fence or a volatile access (both would also wait for the global
+    // stores above); lanes address the cursor by key, so the compiler cannot carry its values across steps
     __builtin_amdgcn_wave_barrier();
-    __threadfence_block();
   }
 }
 
@@ -128,7 +130,15 @@ __device__ inline void block_exclusive_scan(const int *total, int *offsets, int 
 }
 
 // ---- single-block form: everything in one launch -------------------------------------------------
-// Dynamic LDS: hist[kRouteWaves][buckets] + total[buckets] + offsets[buckets+1] + scratch.
+// Dynamic LDS: hist[kRouteWaves][buckets] + total[buckets] + offsets[buckets+1] + scratch + the N keys as 16-bit
+// values.  The kernel runs once per forward on a cold instruction cache, so its loops stay rolled (straight-line
+// code would run at instruction-fetch speed); the keys are read from memory once and kept in LDS for the
+// placement pass.
+__host__ __device__ inline size_t route_single_lds_bytes(int N, int buckets) {
+  size_t ints = (size_t)kRouteWaves * buckets + buckets + buckets + 1 + kRouteWaves + 1;
+  return align_up(ints * sizeof(int), 16) + align_up((size_t)(N > 0 ? N : 1) * sizeof(unsigned short), 16);
+}
+
 template <bool I64>
 __global__ __launch_bounds__(kRouteThreads) void route_single_kernel(
     const void *idx, int N, int E, int capacity, int *sorted_expert, int *sorted_idx, int *counts,
@@ -139,14 +149,32 @@ __global__ __launch_bounds__(kRouteThreads) void route_single_kernel(
   int *total = hist + kRouteWaves * buckets;  // [buckets]
   int *offs = total + buckets;              // [buckets + 1]
   int *scratch = offs + buckets + 1;        // [kRouteWaves + 1]
-  const int tid = threadIdx.x, wave = tid / kWave;
+  unsigned short *keys = (unsigned short *)((char *)lds + align_up(((size_t)kRouteWaves * buckets + 2 * buckets + 1 +
+                                                                   kRouteWaves + 1) * sizeof(int), 16));
+  const int tid = threadIdx.x, wave = tid / kWave, lane = tid & (kWave - 1);
 
   for (int i = tid; i < kRouteWaves * buckets; i += blockDim.x) hist[i] = 0;
   __syncthreads();
 
   int seg = ceil_div(ceil_div(N, kRouteWaves), kWave) * kWave;
   int seg_begin = min(wave * seg, N), seg_end = min(seg_begin + seg, N);
-  wave_histogram<I64>(idx, seg_begin, seg_end, E, hist + wave * buckets);
+  {
+    // four loads in flight per lane; positions past the end are clamped, their keys dropped
+    int *h = hist + wave * buckets;
+    for (int base = seg_begin; base < seg_end; base += 4 * kWave) {
+      int k[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) k[u] = load_key<I64>(idx, min(base + u * kWave + lane, N - 1), E);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        int i = base + u * kWave + lane;
+        if (i < seg_end) {
+          keys[i] = (unsigned short)k[u];
+          atomicAdd(&h[k[u]], 1);
+        }
+      }
+    }
+  }
   __syncthreads();
 
   for (int b = tid; b < buckets; b += blockDim.x) {
@@ -174,8 +202,35 @@ __global__ __launch_bounds__(kRouteThreads) void route_single_kernel(
   }
   __syncthreads();
 
-  wave_place<I64>(idx, seg_begin, seg_end, E, capacity, hist + wave * buckets, offs, sorted_expert,
-                  sorted_idx, inv_pos);
+  // placement, in input order: position = cursor[key] + number of equal keys in lower lanes of the step
+  {
+    int *cursor = hist + wave * buckets;
+    const int key_bits = bits_for(E + 1);
+    const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    for (int base = seg_begin; base < seg_end; base += kWave) {
+      const int i = base + lane;
+      const bool active = i < seg_end;
+      const int k = active ? (int)keys[i] : 0;
+      uint64_t peers = match_key(k, active, key_bits);
+      int rank = __popcll(peers & lt_mask);
+      int start = 0;
+      if (active) start = cursor[k];
+      __builtin_amdgcn_wave_barrier();
+      if (active) {
+        int pos = start + rank;
+        // a valid id is its own key; the rare invalid one is fetched again for the sorted_expert output
+        sorted_expert[pos] = k < E ? k : load_raw<I64>(idx, i);
+        sorted_idx[pos] = i;
+        bool kept = k < E && (pos - offs[k]) < capacity;
+        inv_pos[i] = kept ? pos : -1;
+        if (rank == 0) cursor[k] = start + __popcll(peers);
+      }
+      // the cursor is private to this wave and LDS operations of one wave complete in order: the next step's
+      // read sees this step's write without a fence or a volatile access (both would also wait for the global
+      // stores above); lanes address the cursor by key, so the compiler cannot carry its values across steps
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
 }
 
 // ---- three-kernel form for large N -----------------------------------------------------------
@@ -363,7 +418,18 @@ extern "C" int yamoe_route(const void *router_indices, int32_t idx_i64, int32_t 
   if (capacity < 0) capacity = 0;
   const int buckets = E + 1;
   if (N <= kSingleBlockMaxN) {
-    size_t lds = ((size_t)kRouteWaves * buckets + buckets + buckets + 1 + kRouteWaves + 1) * sizeof(int);
+    size_t lds = route_single_lds_bytes(N, buckets);
+    static bool attr_done = false;  // benign race: the attribute calls are idempotent
+    if (!attr_done) {
+      const int max_lds = (int)route_single_lds_bytes(kSingleBlockMaxN, kRouteMaxBuckets);
+      hipError_t e1 = hipFuncSetAttribute((const void *)route_single_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+      hipError_t e2 = hipFuncSetAttribute((const void *)route_single_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
+      if (e1 != hipSuccess || e2 != hipSuccess) {
+        set_error("hipFuncSetAttribute(MaxDynamicSharedMemorySize=%d): %s", max_lds, hipGetErrorString(e1 != hipSuccess ? e1 : e2));
+        return (int)(e1 != hipSuccess ? e1 : e2);
+      }
+      attr_done = true;
+    }
     if (idx_i64)
       hipLaunchKernelGGL(route_single_kernel<true>, dim3(1), dim3(kRouteThreads), lds, stream,
                          router_indices, N, E, capacity, sorted_expert, sorted_idx, counts, offsets, inv_pos);

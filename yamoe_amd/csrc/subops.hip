@@ -67,7 +67,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_place_kernel(const K *keys,
   for (int i = tid; i < kSortWaves * kRadix; i += kSortThreads)
     cursor_all[i] = seg_cursors[(size_t)blockIdx.x * kSortWaves * kRadix + i];
   __syncthreads();
-  volatile int *cursor = cursor_all + wave * kRadix;
+  int *cursor = cursor_all + wave * kRadix;
   long long seg = (long long)blockIdx.x * kSortWaves + wave;
   long long b = seg * kSortSeg, e = b + kSortSeg;
   if (e > n) e = n;
@@ -93,8 +93,10 @@ __global__ __launch_bounds__(kSortThreads) void sort_place_kernel(const K *keys,
       vals_out[start + rank] = val;
       if (rank == 0) cursor[dg] = start + __popcll(peers);
     }
+    // the cursor is private to this wave and LDS operations of one wave complete in order: the next step's
+    // read sees this step's write without a fence or a volatile access (both would also wait for the global
+    // stores above); lanes address the cursor by key, so the compiler cannot carry its values across steps
     __builtin_amdgcn_wave_barrier();
-    __threadfence_block();
   }
 }
 
