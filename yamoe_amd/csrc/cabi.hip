@@ -227,11 +227,9 @@ static int forward_impl(const yamoe_problem *p, const void *x, const void *idx, 
   const int N = p->T * p->K;
   void *st = (void *)stream;
   if (N == 0 || p->T == 0) return 0;
-  YAMOE_TRY(yamoe_route(idx, p->idx_i64, N, p->E, p->capacity, b.sorted_expert, b.sorted_idx, b.counts, b.offsets,
-                        b.inv_pos, b.route_ws, b.route_ws_bytes, st));
   const int stream_rows = HasStreamPath<T>::value ? kStreamMaxRows : 0;
-  YAMOE_TRY(yamoe_build_schedule(b.counts, b.offsets, N, p->E, p->capacity, stream_rows, b.schedule, b.schedule_bytes,
-                                 st));
+  YAMOE_TRY(route_and_schedule(idx, p->idx_i64, N, p->E, p->capacity, b.sorted_expert, b.sorted_idx, b.counts, b.offsets,
+                               b.inv_pos, b.route_ws, b.route_ws_bytes, stream_rows, b.schedule, b.schedule_bytes, st));
   YAMOE_TRY(tiles_gate_up<T>(x, b.sorted_idx, wgu, bgu, b.act, nullptr, b.schedule, N, p->K, p->E, p->H, p->I, stream));
   if constexpr (HasStreamPath<T>::value)
     YAMOE_TRY(stream_gate_up<T>(x, b.sorted_idx, wgu, bgu, b.act, nullptr, b.schedule, N, p->K, p->E, p->H, p->I,
@@ -261,9 +259,8 @@ static int backward_impl(const yamoe_problem *p, const void *gy, const void *x, 
     YAMOE_TRY(fill_zero(d_bd, (size_t)E * H * es, stream));
     return 0;
   }
-  YAMOE_TRY(yamoe_route(idx, p->idx_i64, N, E, cap, b.f.sorted_expert, b.f.sorted_idx, b.f.counts, b.f.offsets,
-                        b.f.inv_pos, b.f.route_ws, b.f.route_ws_bytes, st));
-  YAMOE_TRY(yamoe_build_schedule(b.f.counts, b.f.offsets, N, E, cap, 0, b.f.schedule, b.f.schedule_bytes, st));
+  YAMOE_TRY(route_and_schedule(idx, p->idx_i64, N, E, cap, b.f.sorted_expert, b.f.sorted_idx, b.f.counts, b.f.offsets,
+                               b.f.inv_pos, b.f.route_ws, b.f.route_ws_bytes, 0, b.f.schedule, b.f.schedule_bytes, st));
   // forward recompute of the first product only: activations and pre-activations
   YAMOE_TRY(launch_permute<T>(x, b.f.sorted_idx, b.x_perm, N, p->K, H, stream));
   YAMOE_TRY(tiles_gate_up<T>(x, b.f.sorted_idx, wgu, bgu, b.f.act, b.pre, b.f.schedule, N, p->K, E, H, I, stream));

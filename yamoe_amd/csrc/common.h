@@ -121,6 +121,11 @@ __host__ __device__ inline ScheduleView schedule_view(const void *p, int N, int 
   return v;
 }
 
+int route_and_schedule(const void *router_indices, int32_t idx_i64, int32_t N, int32_t E, int32_t capacity,
+                       int32_t *sorted_expert, int32_t *sorted_idx, int32_t *counts, int32_t *offsets, int32_t *inv_pos,
+                       void *workspace, size_t workspace_bytes, int32_t stream_max_rows, void *schedule,
+                       size_t schedule_bytes, void *stream);
+
 // error reporting for the C ABI
 void set_error(const char *fmt, ...);
 int check_launch(const char *what);

@@ -129,6 +129,98 @@ __device__ inline void block_exclusive_scan(const int *total, int *offsets, int 
   __syncthreads();
 }
 
+// ---- work lists ------------------------------------------------------------------------------
+// One wave; lane l takes experts l, l+64, ...  Experts with 1..stream_max_rows kept rows go to the
+// streaming list, larger ones are cut into row tiles of kRowTile rows.  Both lists stay in expert
+// order: positions come from wave prefix sums.
+__device__ inline int wave_exclusive_scan(int v, int lane, int &total) {
+  int x = v;
+  for (int d = 1; d < kWave; d <<= 1) {
+    int y = __shfl_up(x, d);
+    if (lane >= d) x += y;
+  }
+  total = __shfl(x, kWave - 1);
+  return x - v;
+}
+
+__device__ inline void build_schedule_wave(const int *counts, const int *offsets, int N, int E, int capacity,
+                                           int stream_max_rows, int *sched, const int lane) {
+  int *row_tiles = sched + kSchedHeader;
+  int *small = row_tiles + 8 * sched_max_row_tiles(N, E);
+  int n_tiles = 0, n_small = 0, n_active = 0, n_kept = 0;
+  for (int base = 0; base < E; base += kWave) {
+    int e = base + lane;
+    int kept = e < E ? min(counts[e], capacity) : 0;
+    if (kept < 0) kept = 0;
+    int first = e < E ? offsets[e] : 0;
+    int is_small = kept > 0 && kept <= stream_max_rows;
+    int tiles = (kept > 0 && !is_small) ? ceil_div(kept, kRowTile) : 0;
+    int tot_small, tot_tiles, tot_active, tot_kept;
+    int pos_small = wave_exclusive_scan(is_small, lane, tot_small);
+    int pos_tiles = wave_exclusive_scan(tiles, lane, tot_tiles);
+    wave_exclusive_scan(kept > 0 ? 1 : 0, lane, tot_active);
+    wave_exclusive_scan(kept, lane, tot_kept);
+    if (is_small) {
+      int *s = small + 4 * (n_small + pos_small);
+      s[0] = e; s[1] = first; s[2] = kept; s[3] = 0;
+    }
+    int gfirst = n_tiles + pos_tiles;
+    // An expert's rows are cut into equal tiles (a multiple of 32 rows, the MFMA block), not into full
+    // tiles plus a remainder: tiles of one expert then advance through the contraction at the same pace
+    // and the weight slabs one of them fetches are still in L2 when the others ask for them.
+    int per_tile = tiles > 0 ? min(kRowTile, (ceil_div(kept, tiles) + 31) & ~31) : 0;
+    for (int t = 0; t < tiles; ++t) {
+      int *w = row_tiles + 8 * (gfirst + t);
+      w[0] = e; w[1] = first + t * per_tile; w[2] = min(per_tile, kept - t * per_tile); w[3] = gfirst; w[4] = tiles;
+      w[5] = 0; w[6] = 0; w[7] = 0;
+    }
+    n_small += tot_small; n_tiles += tot_tiles; n_active += tot_active; n_kept += tot_kept;
+  }
+  // Second pass: cut the tile list into 8 shares of equal cost.  Groups (experts with row tiles) are weighed
+  // by the sum of their tiles' weights; cut x falls into the group that contains x/8 of the total.
+  int w_total = 0;
+  for (int pass = 0; pass < 2; ++pass) {
+    int w_before = 0, t_before = 0;
+    for (int base = 0; base < E; base += kWave) {
+      int e = base + lane;
+      int kept = e < E ? min(counts[e], capacity) : 0;
+      if (kept < 0) kept = 0;
+      int is_small = kept > 0 && kept <= stream_max_rows;
+      int tiles = (kept > 0 && !is_small) ? ceil_div(kept, kRowTile) : 0;
+      int per_tile = tiles > 0 ? min(kRowTile, (ceil_div(kept, tiles) + 31) & ~31) : 0;
+      int w = tiles > 0 ? (tiles - 1) * sched_tile_weight(per_tile) + sched_tile_weight(kept - (tiles - 1) * per_tile) : 0;
+      int tot_w, tot_t;
+      int w_pre = w_before + wave_exclusive_scan(w, lane, tot_w);
+      int t_pre = t_before + wave_exclusive_scan(tiles, lane, tot_t);
+      if (pass == 1 && tiles > 0) {
+        for (int x = 0; x < kXcds; ++x) {
+          long long t = (long long)x * w_total;  // compare x * W / 8 with the group's weight interval, times 8
+          if (t >= 8ll * w_pre && t < 8ll * (w_pre + w)) {
+            int *c = sched + kSchedCuts + 4 * x;
+            c[0] = t_pre; c[1] = (int)(((t - 8ll * w_pre) << 16) / (8ll * w)); c[2] = 0; c[3] = tiles;
+          }
+        }
+      }
+      w_before += tot_w; t_before += tot_t;
+    }
+    if (pass == 0) w_total = w_before;
+  }
+  if (lane == 0) {
+    sched[0] = n_tiles; sched[1] = n_small; sched[2] = n_active; sched[3] = n_kept;
+    sched[4] = w_total; sched[5] = 0; sched[6] = 0; sched[7] = 0;
+    int *c = sched + kSchedCuts + 4 * kXcds;  // the end of the list
+    c[0] = n_tiles; c[1] = 0; c[2] = 0; c[3] = 0;
+    if (w_total == 0)
+      for (int x = 0; x < kXcds; ++x) { int *cx = sched + kSchedCuts + 4 * x; cx[0] = 0; cx[1] = 0; cx[2] = 0; cx[3] = 0; }
+    for (int i = kSchedCuts + 4 * (kXcds + 1); i < kSchedHeader; ++i) sched[i] = 0;
+  }
+}
+
+__global__ __launch_bounds__(kWave) void build_schedule_kernel(const int *counts, const int *offsets, int N, int E,
+                                                               int capacity, int stream_max_rows, int *sched) {
+  build_schedule_wave(counts, offsets, N, E, capacity, stream_max_rows, sched, threadIdx.x);
+}
+
 // ---- single-block form: everything in one launch -------------------------------------------------
 // Dynamic LDS: hist[kRouteWaves][buckets] + total[buckets] + offsets[buckets+1] + scratch + the N keys as 16-bit
 // values.  The kernel runs once per forward on a cold instruction cache, so its loops stay rolled (straight-line
@@ -142,7 +234,7 @@ __host__ __device__ inline size_t route_single_lds_bytes(int N, int buckets) {
 template <bool I64>
 __global__ __launch_bounds__(kRouteThreads) void route_single_kernel(
     const void *idx, int N, int E, int capacity, int *sorted_expert, int *sorted_idx, int *counts,
-    int *offsets_out, int *inv_pos) {
+    int *offsets_out, int *inv_pos, int *sched, int stream_max_rows) {
   extern __shared__ int lds[];
   const int buckets = E + 1;
   int *hist = lds;                          // [kRouteWaves][buckets]
@@ -231,6 +323,9 @@ __global__ __launch_bounds__(kRouteThreads) void route_single_kernel(
       __builtin_amdgcn_wave_barrier();
     }
   }
+  // the work lists of the GEMM kernels, from the counts and offsets still in LDS (the last wave, after its share
+  // of the placement): saves the launch of build_schedule_kernel
+  if (sched != nullptr && wave == kRouteWaves - 1) build_schedule_wave(total, offs, N, E, capacity, stream_max_rows, sched, lane);
 }
 
 // ---- three-kernel form for large N -----------------------------------------------------------
@@ -303,94 +398,6 @@ __global__ __launch_bounds__(kRouteThreads) void route_place_kernel(
                   inv_pos);
 }
 
-// ---- work lists ------------------------------------------------------------------------------
-// One wave; lane l takes experts l, l+64, ...  Experts with 1..stream_max_rows kept rows go to the
-// streaming list, larger ones are cut into row tiles of kRowTile rows.  Both lists stay in expert
-// order: positions come from wave prefix sums.
-__device__ inline int wave_exclusive_scan(int v, int lane, int &total) {
-  int x = v;
-  for (int d = 1; d < kWave; d <<= 1) {
-    int y = __shfl_up(x, d);
-    if (lane >= d) x += y;
-  }
-  total = __shfl(x, kWave - 1);
-  return x - v;
-}
-
-__global__ __launch_bounds__(kWave) void build_schedule_kernel(const int *counts, const int *offsets, int N, int E,
-                                                               int capacity, int stream_max_rows, int *sched) {
-  const int lane = threadIdx.x;
-  int *row_tiles = sched + kSchedHeader;
-  int *small = row_tiles + 8 * sched_max_row_tiles(N, E);
-  int n_tiles = 0, n_small = 0, n_active = 0, n_kept = 0;
-  for (int base = 0; base < E; base += kWave) {
-    int e = base + lane;
-    int kept = e < E ? min(counts[e], capacity) : 0;
-    if (kept < 0) kept = 0;
-    int first = e < E ? offsets[e] : 0;
-    int is_small = kept > 0 && kept <= stream_max_rows;
-    int tiles = (kept > 0 && !is_small) ? ceil_div(kept, kRowTile) : 0;
-    int tot_small, tot_tiles, tot_active, tot_kept;
-    int pos_small = wave_exclusive_scan(is_small, lane, tot_small);
-    int pos_tiles = wave_exclusive_scan(tiles, lane, tot_tiles);
-    wave_exclusive_scan(kept > 0 ? 1 : 0, lane, tot_active);
-    wave_exclusive_scan(kept, lane, tot_kept);
-    if (is_small) {
-      int *s = small + 4 * (n_small + pos_small);
-      s[0] = e; s[1] = first; s[2] = kept; s[3] = 0;
-    }
-    int gfirst = n_tiles + pos_tiles;
-    // An expert's rows are cut into equal tiles (a multiple of 32 rows, the MFMA block), not into full
-    // tiles plus a remainder: tiles of one expert then advance through the contraction at the same pace
-    // and the weight slabs one of them fetches are still in L2 when the others ask for them.
-    int per_tile = tiles > 0 ? min(kRowTile, (ceil_div(kept, tiles) + 31) & ~31) : 0;
-    for (int t = 0; t < tiles; ++t) {
-      int *w = row_tiles + 8 * (gfirst + t);
-      w[0] = e; w[1] = first + t * per_tile; w[2] = min(per_tile, kept - t * per_tile); w[3] = gfirst; w[4] = tiles;
-      w[5] = 0; w[6] = 0; w[7] = 0;
-    }
-    n_small += tot_small; n_tiles += tot_tiles; n_active += tot_active; n_kept += tot_kept;
-  }
-  // Second pass: cut the tile list into 8 shares of equal cost.  Groups (experts with row tiles) are weighed
-  // by the sum of their tiles' weights; cut x falls into the group that contains x/8 of the total.
-  int w_total = 0;
-  for (int pass = 0; pass < 2; ++pass) {
-    int w_before = 0, t_before = 0;
-    for (int base = 0; base < E; base += kWave) {
-      int e = base + lane;
-      int kept = e < E ? min(counts[e], capacity) : 0;
-      if (kept < 0) kept = 0;
-      int is_small = kept > 0 && kept <= stream_max_rows;
-      int tiles = (kept > 0 && !is_small) ? ceil_div(kept, kRowTile) : 0;
-      int per_tile = tiles > 0 ? min(kRowTile, (ceil_div(kept, tiles) + 31) & ~31) : 0;
-      int w = tiles > 0 ? (tiles - 1) * sched_tile_weight(per_tile) + sched_tile_weight(kept - (tiles - 1) * per_tile) : 0;
-      int tot_w, tot_t;
-      int w_pre = w_before + wave_exclusive_scan(w, lane, tot_w);
-      int t_pre = t_before + wave_exclusive_scan(tiles, lane, tot_t);
-      if (pass == 1 && tiles > 0) {
-        for (int x = 0; x < kXcds; ++x) {
-          long long t = (long long)x * w_total;  // compare x * W / 8 with the group's weight interval, times 8
-          if (t >= 8ll * w_pre && t < 8ll * (w_pre + w)) {
-            int *c = sched + kSchedCuts + 4 * x;
-            c[0] = t_pre; c[1] = (int)(((t - 8ll * w_pre) << 16) / (8ll * w)); c[2] = 0; c[3] = tiles;
-          }
-        }
-      }
-      w_before += tot_w; t_before += tot_t;
-    }
-    if (pass == 0) w_total = w_before;
-  }
-  if (lane == 0) {
-    sched[0] = n_tiles; sched[1] = n_small; sched[2] = n_active; sched[3] = n_kept;
-    sched[4] = w_total; sched[5] = 0; sched[6] = 0; sched[7] = 0;
-    int *c = sched + kSchedCuts + 4 * kXcds;  // the end of the list
-    c[0] = n_tiles; c[1] = 0; c[2] = 0; c[3] = 0;
-    if (w_total == 0)
-      for (int x = 0; x < kXcds; ++x) { int *cx = sched + kSchedCuts + 4 * x; cx[0] = 0; cx[1] = 0; cx[2] = 0; cx[3] = 0; }
-    for (int i = kSchedCuts + 4 * (kXcds + 1); i < kSchedHeader; ++i) sched[i] = 0;
-  }
-}
-
 }  // namespace yamoe
 
 using namespace yamoe;
@@ -402,11 +409,19 @@ extern "C" size_t yamoe_route_workspace_bytes(int32_t N, int32_t E) {
   return align_up((size_t)n_seg * (E + 1) * sizeof(int), 256);
 }
 
-extern "C" int yamoe_route(const void *router_indices, int32_t idx_i64, int32_t N, int32_t E,
-                           int32_t capacity, int32_t *sorted_expert, int32_t *sorted_idx,
-                           int32_t *counts, int32_t *offsets, int32_t *inv_pos, void *workspace,
-                           size_t workspace_bytes, void *stream_) {
+// yamoe_route, optionally followed by yamoe_build_schedule (schedule != nullptr); for N up to kSingleBlockMaxN both
+// run in one launch.
+int yamoe::route_and_schedule(const void *router_indices, int32_t idx_i64, int32_t N, int32_t E, int32_t capacity,
+                              int32_t *sorted_expert, int32_t *sorted_idx, int32_t *counts, int32_t *offsets,
+                              int32_t *inv_pos, void *workspace, size_t workspace_bytes, int32_t stream_max_rows,
+                              void *schedule, size_t schedule_bytes, void *stream_) {
   hipStream_t stream = (hipStream_t)stream_;
+  if (schedule != nullptr && schedule_bytes < yamoe_schedule_bytes(N, E)) {
+    set_error("yamoe_build_schedule: schedule region too small");
+    return YAMOE_E_WORKSPACE;
+  }
+  if (stream_max_rows < 0) stream_max_rows = 0;
+  if (stream_max_rows > kStreamMaxRows) stream_max_rows = kStreamMaxRows;
   if (N < 0 || E <= 0 || E + 1 > kRouteMaxBuckets) {
     set_error("yamoe_route: need N >= 0 and 1 <= E < %d (got N=%d E=%d)", kRouteMaxBuckets, N, E);
     return YAMOE_E_ARG;
@@ -432,10 +447,12 @@ extern "C" int yamoe_route(const void *router_indices, int32_t idx_i64, int32_t 
     }
     if (idx_i64)
       hipLaunchKernelGGL(route_single_kernel<true>, dim3(1), dim3(kRouteThreads), lds, stream,
-                         router_indices, N, E, capacity, sorted_expert, sorted_idx, counts, offsets, inv_pos);
+                         router_indices, N, E, capacity, sorted_expert, sorted_idx, counts, offsets, inv_pos, (int *)schedule,
+                         stream_max_rows);
     else
       hipLaunchKernelGGL(route_single_kernel<false>, dim3(1), dim3(kRouteThreads), lds, stream,
-                         router_indices, N, E, capacity, sorted_expert, sorted_idx, counts, offsets, inv_pos);
+                         router_indices, N, E, capacity, sorted_expert, sorted_idx, counts, offsets, inv_pos, (int *)schedule,
+                         stream_max_rows);
     return check_launch("route_single_kernel");
   }
   if (workspace_bytes < yamoe_route_workspace_bytes(N, E) || !workspace) {
@@ -467,7 +484,17 @@ extern "C" int yamoe_route(const void *router_indices, int32_t idx_i64, int32_t 
   else
     hipLaunchKernelGGL(route_place_kernel<false>, dim3(n_blocks), dim3(kRouteThreads), lds_c, stream,
                        router_indices, N, E, capacity, seg, seg_counts, offsets, sorted_expert, sorted_idx, inv_pos);
-  return check_launch("route_place_kernel");
+  rc = check_launch("route_place_kernel");
+  if (rc || schedule == nullptr) return rc;
+  return yamoe_build_schedule(counts, offsets, N, E, capacity, stream_max_rows, schedule, schedule_bytes, stream_);
+}
+
+extern "C" int yamoe_route(const void *router_indices, int32_t idx_i64, int32_t N, int32_t E,
+                           int32_t capacity, int32_t *sorted_expert, int32_t *sorted_idx,
+                           int32_t *counts, int32_t *offsets, int32_t *inv_pos, void *workspace,
+                           size_t workspace_bytes, void *stream_) {
+  return route_and_schedule(router_indices, idx_i64, N, E, capacity, sorted_expert, sorted_idx, counts, offsets, inv_pos,
+                            workspace, workspace_bytes, 0, nullptr, 0, stream_);
 }
 
 extern "C" size_t yamoe_schedule_bytes(int32_t N, int32_t E) {
