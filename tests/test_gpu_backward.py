@@ -48,6 +48,24 @@ def test_backward_small(gpu, dtype, T, H, I, E, K):
     check(grads, want, dtype, "small")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("capacity", [200, 37, 600])
+def test_backward_capacity_16bit(gpu, dtype, capacity):
+    """Dropped assignments on the 16-bit kernels: the weight-gradient contraction stops at the capacity (200 rows: a
+    partial last slab on the pipelined path; 37: the short path), the input-gradient GEMM gathers grad_out by token
+    only for kept rows, dropped slots get a zero routing gradient."""
+    T, H, I, E, K = 600, 128, 64, 4, 2
+    d = make_inputs(T, H, I, E, K, dtype, seed=9, w_std=0.05, bias_std=0.1, zipf=0.5)
+    gy = torch.randn(T, H, generator=torch.Generator().manual_seed(3)).to(dtype)
+    grads = run_bwd(d, gy, capacity, gpu)
+    want = O.experts_backward(gy, *args(d), capacity, compute_dtype=torch.float32)
+    check(grads, want, dtype, "capacity %d" % capacity)
+    r = O.route(d["router_indices"], E, capacity)
+    dropped = torch.from_numpy(r["inv_pos"].reshape(T, K) < 0)
+    d_routing = grads[1].cpu()
+    assert torch.all(torch.gather(d_routing, 1, d["router_indices"])[dropped] == 0)
+
+
 @pytest.mark.parametrize("slot_weights", [False, True])
 def test_backward_capacity_and_layouts(gpu, slot_weights):
     dtype = torch.float32

@@ -80,6 +80,17 @@ def test_forward_uneven_tile_costs(gpu):
     assert report("uneven tile costs", got.double(), want.double(), tol) < tol
 
 
+def test_forward_many_assignments(gpu):
+    """N = T*K above the single-workgroup routing limit (32 768): three-kernel routing, separate work-list launch,
+    skewed expert loads with some experts empty."""
+    T, H, I, E, K = 20000, 128, 64, 16, 2
+    d = make_inputs(T, H, I, E, K, torch.bfloat16, seed=21, w_std=0.05, bias_std=0.1, zipf=1.2)
+    got = run_op(d, T, gpu)
+    want = oracle_forward(d, T)
+    tol = REL_L2_TOL[torch.bfloat16]
+    assert report("many assignments", got.double(), want.double(), tol) < tol
+
+
 def test_forward_special_cases(gpu):
     """Structure checks that do not depend on the oracle's matmul: one-hot routing returns the
     expert's row, zero weights reduce to the bias closed form, an unused expert changes nothing."""
