@@ -170,14 +170,37 @@ __global__ __launch_bounds__(kRowThreads) void glu_backward_rows_kernel(
     const T *pr = pre + (size_t)p * 2 * I;
     T *dp = d_pre + (size_t)p * 2 * I;
     float dot = 0.0f;
-    for (int c = lane; c < I; c += kWave) {
-      float G = ElemTraits<T>::to_f32(pr[2 * c]), U = ElemTraits<T>::to_f32(pr[2 * c + 1]);
-      float dh = ElemTraits<T>::to_f32(da[c]);
-      float dG, dU;
-      glu_backward(G, U, dh * w, dG, dU);
-      dot += dh * glu_forward(G, U);
-      dp[2 * c] = ElemTraits<T>::from_f32(dG);
-      dp[2 * c + 1] = ElemTraits<T>::from_f32(dU);
+    constexpr int V = ElemTraits<T>::kVec;  // pre-activations per 16 bytes = V / 2 (gate, up) pairs
+    if (I % (V / 2) == 0) {
+      for (int c = lane; c < I / (V / 2); c += kWave) {
+        u32x4 praw = ((const u32x4 *)pr)[c];
+        u32x2 draw = ((const u32x2 *)da)[c];
+        const T *pv = (const T *)&praw;
+        const T *dv = (const T *)&draw;
+        u32x4 oraw;
+        T *ov = (T *)&oraw;
+#pragma unroll
+        for (int j = 0; j < V / 2; ++j) {
+          float G = ElemTraits<T>::to_f32(pv[2 * j]), U = ElemTraits<T>::to_f32(pv[2 * j + 1]);
+          float dh = ElemTraits<T>::to_f32(dv[j]);
+          float dG, dU;
+          glu_backward(G, U, dh * w, dG, dU);
+          dot += dh * glu_forward(G, U);
+          ov[2 * j] = ElemTraits<T>::from_f32(dG);
+          ov[2 * j + 1] = ElemTraits<T>::from_f32(dU);
+        }
+        ((u32x4 *)dp)[c] = oraw;
+      }
+    } else {
+      for (int c = lane; c < I; c += kWave) {
+        float G = ElemTraits<T>::to_f32(pr[2 * c]), U = ElemTraits<T>::to_f32(pr[2 * c + 1]);
+        float dh = ElemTraits<T>::to_f32(da[c]);
+        float dG, dU;
+        glu_backward(G, U, dh * w, dG, dU);
+        dot += dh * glu_forward(G, U);
+        dp[2 * c] = ElemTraits<T>::from_f32(dG);
+        dp[2 * c + 1] = ElemTraits<T>::from_f32(dU);
+      }
     }
     for (int d = kWave / 2; d > 0; d >>= 1) dot += __shfl_xor(dot, d);
     if (lane == 0) {
