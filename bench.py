@@ -256,7 +256,18 @@ def main():
         timed(lambda: yamoe_amd.experts(*az, zc["T"], zc["E"], zc["K"]), zc["T"] * zc["K"] * 6 * H * I,
               "forward_zipf_bf16")
         cz = np.bincount(hostz["router_indices"].numpy().ravel(), minlength=zc["E"])
-        extras["forward_zipf_bf16"].update(max_rows=int(cz.max()), empty_experts=int((cz == 0).sum()))
+        n_z = zc["T"] * zc["K"]
+        w_bytes = int((cz > 0).sum()) * 3 * H * I * 2               # weights of the non-empty experts, read once
+        roof_ms = max(n_z * 6 * H * I / (PEAK_BF16_TFLOPS * 1e12), w_bytes / (PEAK_HBM_GBS * 1e9)) * 1e3
+        extras["forward_zipf_bf16"].update(max_rows=int(cz.max()), empty_experts=int((cz == 0).sum()),
+                                           roofline_ms=round(roof_ms, 4))
+        # its routing kernels (three launches at this N) and the row permute on their own
+        r_ms = event_time_ms(lambda: _cabi.route(dz["router_indices"], zc["E"], zc["T"]), 50)
+        se_z, si_z, _, _, _ = _cabi.route(dz["router_indices"], zc["E"], zc["T"])
+        p_ms = event_time_ms(lambda: _cabi.permute(dz["hidden"], si_z, zc["K"]), 50)
+        extras["routing_zipf"] = dict(assignments=n_z, route_ms=round(r_ms, 4), permute_ms=round(p_ms, 4),
+                                      permute_gbs=round((2 * n_z * H * 2 + 4 * n_z) / (p_ms * 1e-3) / 1e9, 1))
+        del se_z, si_z
         del dz, az
         torch.cuda.empty_cache()
         # README shape, fp32 (peak 157.3 TFLOP/s fp32 MFMA)
