@@ -116,3 +116,21 @@ def test_workloads_are_seeded_and_shaped():
     counts = torch.bincount(z["router_indices"].flatten(), minlength=128)
     assert counts.max() > 10 * counts.float().mean() and (counts == 0).any()
     assert set(CONFIGS) == {"readme", "gptoss20b", "decode", "zipf"}
+
+
+def test_hub_layout_imports_as_yamoe(tmp_path):
+    """`python -m yamoe_amd.package` lays out build/<variant>/yamoe/ (the reference's hub layout, build.toml:1-36);
+    that directory imports as `yamoe` with the reference's names.  Run in a child process: the operator library
+    registers its ops once per process."""
+    import subprocess
+    import sys
+    from yamoe_amd import package
+    dst = package.package(str(tmp_path))
+    assert os.path.basename(dst) == "yamoe" and re.match(r"torch\d+-cxx11-rocm\d+-x86_64-linux$", os.path.basename(os.path.dirname(dst)))
+    assert 'backend = "rocm"' in open(os.path.join(str(tmp_path), "build.toml")).read()
+    code = ("import sys; sys.path.insert(0, %r); import yamoe; "
+            "names = ['experts', 'experts_backward', 'gather', 'scatter', 'sort', 'bincount_cumsum', 'batch_mm', 'ops', 'Yamoe']; "
+            "assert all(getattr(yamoe, n) is not None for n in names); "
+            "assert 'yamoe_amd' not in sys.modules; print('ok')" % os.path.dirname(dst))
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, cwd=str(tmp_path))
+    assert r.returncode == 0 and r.stdout.strip().endswith("ok"), r.stderr[-2000:]

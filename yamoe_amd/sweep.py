@@ -46,7 +46,7 @@ def make_point(batch_size, seq_len, hidden_dim, num_experts, top_k, dtype=torch.
 
 
 def run_point(batch_size, seq_len, hidden_dim, num_experts, top_k, iters=20, warmup=5, capacity="tokens", dtype=torch.float16):
-    import yamoe_amd
+    from . import experts
     p = make_point(batch_size, seq_len, hidden_dim, num_experts, top_k, dtype)
     tokens = batch_size * seq_len
     cap = seq_len if capacity == "seq" else tokens
@@ -55,14 +55,14 @@ def run_point(batch_size, seq_len, hidden_dim, num_experts, top_k, iters=20, war
     counts = torch.bincount(p["router_indices"].reshape(-1), minlength=num_experts)
     kept = int(torch.clamp(counts, max=cap).sum())
     for _ in range(warmup):
-        yamoe_amd.experts(*args)
+        experts(*args)
     torch.cuda.synchronize()
     torch.cuda.reset_peak_memory_stats()
     before = torch.cuda.memory_allocated()
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for _ in range(iters):
-        out = yamoe_amd.experts(*args)
+        out = experts(*args)
     end.record()
     torch.cuda.synchronize()
     ms = start.elapsed_time(end) / iters
