@@ -164,3 +164,39 @@ def test_sweep_point_runs(gpu):
     r = sweep.run_point(2, 64, 128, 8, 2, iters=2, warmup=1, capacity="seq")
     assert r["kept_assignments"] <= 2 * 64 * 2 and r["capacity"] == 64
     assert len(sweep.CONFIGS) == 6 and sweep.BATCH_SIZES == [1, 2, 4, 8, 16, 32, 64]
+
+
+def test_forward_and_backward_replay_in_a_hip_graph(gpu):
+    """The op makes no host synchronisation and no memset node: captured once into a graph and replayed with
+    other work in between, every replay reproduces the eager result bit for bit."""
+    import yamoe_amd
+    T, H, I, E, K = 700, 128, 128, 8, 2
+    d = make_inputs(T, H, I, E, K, torch.bfloat16, seed=31, w_std=0.05, bias_std=0.1, zipf=0.7)
+    g = to_dev(d, gpu)
+    gy = torch.randn(T, H, generator=torch.Generator().manual_seed(4)).to(torch.bfloat16).to(gpu)
+    a = args(g)
+    eager_out = yamoe_amd.experts(*a, T, E, K)
+    eager_grads = yamoe_amd.experts_backward(gy, *a, T, E, K)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for _ in range(2):                                    # warm-up on the capture stream
+            yamoe_amd.experts(*a, T, E, K)
+            yamoe_amd.experts_backward(gy, *a, T, E, K)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        out = yamoe_amd.experts(*a, T, E, K)
+        grads = yamoe_amd.experts_backward(gy, *a, T, E, K)
+    for rep in range(3):
+        out.zero_()
+        for t in grads:
+            t.fill_(7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager_out), rep
+        for got, want in zip(grads, eager_grads):
+            assert torch.equal(got, want), rep
+        yamoe_amd.experts(*a, T, E, K)                        # eager work between replays
+        torch.cuda.synchronize()
