@@ -122,6 +122,15 @@ def test_forward_gptoss20b_full(gpu):
     assert O.rel_l2(half.float() * 2, got.float()) < 1e-2
 
 
+def test_forward_gptoss20b_full_fp16(gpu):
+    """The same layer in fp16 (the dtype of the reference's timing sweep, perf_plot.py:93-101)."""
+    d, c = make_config("gptoss20b", seed=3)
+    d = {k: (v.to(torch.float16) if v.is_floating_point() else v) for k, v in d.items()}
+    got = run_op(d, c["T"], gpu)
+    want = oracle_forward(d, c["T"])
+    assert report("gptoss20b fp16", got, want, 1e-2) < 1e-2
+
+
 def test_forward_decode_full_rows(gpu):
     """Decode regime at the real expert shape (fewer experts to keep host generation short)."""
     d = make_inputs(64, 2880, 2880, 32, 4, torch.bfloat16, seed=5)
