@@ -56,9 +56,10 @@ int stream_down(const void *, const void *, const void *, void *, const void *, 
 
 template <typename T>
 int gemm_async_gate_up(const void *, const int *, const void *, const void *, void *, void *, const void *, int, int,
-                       int, int, int, hipStream_t);
+                       int, int, int, int, hipStream_t);
 template <typename T>
-int gemm_async_down(const void *, const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);
+int gemm_async_down(const void *, const void *, const void *, void *, const void *, int, int, int, int, int,
+                    hipStream_t);
 template <typename T>
 int gemm_async_dgrad(const void *, const int *, int, const void *, void *, const void *, int, int, int, int,
                      hipStream_t);
@@ -72,20 +73,23 @@ template <typename T> struct HasStreamPath { static constexpr bool value = sizeo
 // The MFMA tile kernels for the two forward products: the asynchronous-copy pipeline when the dtype
 // and shape allow it, the register-staged kernel otherwise.
 template <typename T>
+// `small_rows`: experts with at most this many kept rows are on the schedule's streaming list, not tiled (0 when
+// unknown); it only tightens the grid.
 static int tiles_gate_up(const void *x, const int *sorted_idx, const void *w, const void *bias, void *act, void *pre,
-                         const void *sched, int N, int K, int E, int H, int I, hipStream_t stream) {
+                         const void *sched, int N, int K, int E, int H, int I, int small_rows, hipStream_t stream) {
   if constexpr (sizeof(T) == 2) {
     // the gathered source rows span the whole hidden_states tensor: N / K tokens of H elements
     if (gemm_async_supported(H, 2 * I, H, 2 * I, (long long)(N / K) * H * (long long)sizeof(T)))
-      return gemm_async_gate_up<T>(x, sorted_idx, w, bias, act, pre, sched, N, K, E, H, I, stream);
+      return gemm_async_gate_up<T>(x, sorted_idx, w, bias, act, pre, sched, N, K, E, H, I, small_rows, stream);
   }
   return gemm_gate_up<T>(x, sorted_idx, w, bias, act, pre, sched, N, K, E, H, I, stream);
 }
 template <typename T>
 static int tiles_down(const void *act, const void *w, const void *bias, void *y, const void *sched, int N, int E,
-                      int H, int I, hipStream_t stream) {
+                      int H, int I, int small_rows, hipStream_t stream) {
   if constexpr (sizeof(T) == 2) {
-    if (gemm_async_supported(I, H, I, H, 0)) return gemm_async_down<T>(act, w, bias, y, sched, N, E, H, I, stream);
+    if (gemm_async_supported(I, H, I, H, 0))
+      return gemm_async_down<T>(act, w, bias, y, sched, N, E, H, I, small_rows, stream);
   }
   return gemm_down<T>(act, w, bias, y, sched, N, E, H, I, stream);
 }
@@ -230,11 +234,12 @@ static int forward_impl(const yamoe_problem *p, const void *x, const void *idx, 
   const int stream_rows = HasStreamPath<T>::value ? kStreamMaxRows : 0;
   YAMOE_TRY(route_and_schedule(idx, p->idx_i64, N, p->E, p->capacity, b.sorted_expert, b.sorted_idx, b.counts, b.offsets,
                                b.inv_pos, b.route_ws, b.route_ws_bytes, stream_rows, b.schedule, b.schedule_bytes, st));
-  YAMOE_TRY(tiles_gate_up<T>(x, b.sorted_idx, wgu, bgu, b.act, nullptr, b.schedule, N, p->K, p->E, p->H, p->I, stream));
+  YAMOE_TRY(tiles_gate_up<T>(x, b.sorted_idx, wgu, bgu, b.act, nullptr, b.schedule, N, p->K, p->E, p->H, p->I, stream_rows,
+                             stream));
   if constexpr (HasStreamPath<T>::value)
     YAMOE_TRY(stream_gate_up<T>(x, b.sorted_idx, wgu, bgu, b.act, nullptr, b.schedule, N, p->K, p->E, p->H, p->I,
                                 stream));
-  YAMOE_TRY(tiles_down<T>(b.act, wd, bd, b.y_perm, b.schedule, N, p->E, p->H, p->I, stream));
+  YAMOE_TRY(tiles_down<T>(b.act, wd, bd, b.y_perm, b.schedule, N, p->E, p->H, p->I, stream_rows, stream));
   if constexpr (HasStreamPath<T>::value)
     YAMOE_TRY(stream_down<T>(b.act, wd, bd, b.y_perm, b.schedule, N, p->E, p->H, p->I, stream));
   YAMOE_TRY(launch_combine<T>(b.y_perm, b.inv_pos, idx, p->idx_i64, rw, p->rw_cols, out, p->T, p->K, p->E, p->H,
@@ -263,7 +268,7 @@ static int backward_impl(const yamoe_problem *p, const void *gy, const void *x, 
                                b.f.inv_pos, b.f.route_ws, b.f.route_ws_bytes, 0, b.f.schedule, b.f.schedule_bytes, st));
   // forward recompute of the first product only: activations and pre-activations
   YAMOE_TRY(launch_permute<T>(x, b.f.sorted_idx, b.x_perm, N, p->K, H, stream));
-  YAMOE_TRY(tiles_gate_up<T>(x, b.f.sorted_idx, wgu, bgu, b.f.act, b.pre, b.f.schedule, N, p->K, E, H, I, stream));
+  YAMOE_TRY(tiles_gate_up<T>(x, b.f.sorted_idx, wgu, bgu, b.f.act, b.pre, b.f.schedule, N, p->K, E, H, I, 0, stream));
   // combine backward: g_y_perm = grad_out[tok] * w, and the bias part of the routing gradient
   YAMOE_TRY(launch_combine_backward<T>(gy, bd, b.f.sorted_idx, b.f.inv_pos, idx, p->idx_i64, rw, p->rw_cols, b.g_y_perm,
                                        b.w_sorted, b.dot_bias, N, p->K, E, H, stream));
@@ -317,7 +322,7 @@ static int check_gemm_shape(const char *who, int N, int E, int H, int I, int dty
 template <typename T>
 static int gate_up_both(const void *x, const int *sorted_idx, const void *w, const void *bias, void *act, void *pre,
                         const void *sched, int N, int K, int E, int H, int I, hipStream_t stream) {
-  YAMOE_TRY(tiles_gate_up<T>(x, sorted_idx, w, bias, act, pre, sched, N, K, E, H, I, stream));
+  YAMOE_TRY(tiles_gate_up<T>(x, sorted_idx, w, bias, act, pre, sched, N, K, E, H, I, 0, stream));
   if constexpr (HasStreamPath<T>::value)
     YAMOE_TRY(stream_gate_up<T>(x, sorted_idx, w, bias, act, pre, sched, N, K, E, H, I, stream));
   return 0;
@@ -325,7 +330,7 @@ static int gate_up_both(const void *x, const int *sorted_idx, const void *w, con
 template <typename T>
 static int down_both(const void *act, const void *w, const void *bias, void *y, const void *sched, int N, int E, int H,
                      int I, hipStream_t stream) {
-  YAMOE_TRY(tiles_down<T>(act, w, bias, y, sched, N, E, H, I, stream));
+  YAMOE_TRY(tiles_down<T>(act, w, bias, y, sched, N, E, H, I, 0, stream));
   if constexpr (HasStreamPath<T>::value) YAMOE_TRY(stream_down<T>(act, w, bias, y, sched, N, E, H, I, stream));
   return 0;
 }

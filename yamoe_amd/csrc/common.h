@@ -105,6 +105,13 @@ __host__ __device__ inline int sched_max_row_tiles(int N, int E) {
   // every expert with kept rows adds at most one partly filled tile
   return N / kRowTile + (N < E ? N : E) + 1;
 }
+// Upper bound of the row-tile count when experts with at most `small_rows` kept rows are not tiled (they are on
+// the streaming list): only N / (small_rows + 1) experts can hold more rows than that.  Used for grid sizes only.
+__host__ __device__ inline int sched_grid_row_tiles(int N, int E, int small_rows) {
+  int tiled = N / (small_rows + 1);
+  if (tiled > E) tiled = E;
+  return N / kRowTile + tiled + 1;
+}
 __host__ __device__ inline int sched_max_small(int N, int E) { return (N < E ? N : E) + 1; }
 
 struct ScheduleView {

@@ -785,25 +785,25 @@ bool gemm_async_supported(int Kd, int Nd, int lda, int ldb, long long a_span_byt
 
 template <typename T>
 int gemm_async_gate_up(const void *x, const int *sorted_idx, const void *w, const void *bias, void *act, void *pre,
-                       const void *sched, int N, int K, int E, int H, int I, hipStream_t stream) {
+                       const void *sched, int N, int K, int E, int H, int I, int small_rows, hipStream_t stream) {
   async::Args a = {};
   a.A = x; a.B = w; a.bias = bias; a.C = act; a.C2 = pre;
   a.a_rows = sorted_idx; a.a_div = K; a.sched = (const int *)sched;
   a.Kd = H; a.Nd = 2 * I; a.lda = H; a.ldb = 2 * I; a.ldc = I;
   a.b_expert_stride = (long long)H * 2 * I;
   a.n_col_tiles = ceil_div(2 * I, async::kBN);
-  return async::launch<T, async::EPI_GLU, true, false>(a, sched_max_row_tiles(N, E), stream);
+  return async::launch<T, async::EPI_GLU, true, false>(a, sched_grid_row_tiles(N, E, small_rows), stream);
 }
 
 template <typename T>
 int gemm_async_down(const void *act, const void *w, const void *bias, void *y, const void *sched, int N, int E, int H,
-                    int I, hipStream_t stream) {
+                    int I, int small_rows, hipStream_t stream) {
   async::Args a = {};
   a.A = act; a.B = w; a.bias = bias; a.C = y; a.sched = (const int *)sched;
   a.Kd = I; a.Nd = H; a.lda = I; a.ldb = H; a.ldc = H;
   a.b_expert_stride = (long long)I * H;
   a.n_col_tiles = ceil_div(H, async::kBN);
-  return async::launch<T, async::EPI_STORE, false, false>(a, sched_max_row_tiles(N, E), stream);
+  return async::launch<T, async::EPI_STORE, false, false>(a, sched_grid_row_tiles(N, E, small_rows), stream);
 }
 
 // C[rows, Nd] = A[rows, Kd] * W[e]^T with W[e] stored [Nd, Kd]: the input gradients of both projections
@@ -853,9 +853,9 @@ int gemm_async_wgrad(const void *L, const void *R, void *dW, const int *counts, 
 
 #define YAMOE_INSTANTIATE_ASYNC(T)                                                                               \
   template int gemm_async_gate_up<T>(const void *, const int *, const void *, const void *, void *, void *,      \
-                                     const void *, int, int, int, int, int, hipStream_t);                        \
+                                     const void *, int, int, int, int, int, int, hipStream_t);                   \
   template int gemm_async_down<T>(const void *, const void *, const void *, void *, const void *, int, int, int, \
-                                  int, hipStream_t);                                                             \
+                                  int, int, hipStream_t);                                                             \
   template int gemm_async_dgrad<T>(const void *, const int *, int, const void *, void *, const void *, int, int, int,  \
                                    int, hipStream_t);                                                                  \
   template int gemm_async_wgrad<T>(const void *, const void *, void *, const int *, const int *, int, int, int, int,    \
