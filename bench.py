@@ -26,6 +26,9 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+# the headline metric this file reports: `value` is its first part (forward TFLOP/s of the 20B shape), the `decode`
+# object on the same line carries the second (GB/s and fraction of HBM peak)
+METRIC = "experts() fwd TFLOP/s & %MFMA peak (20B shape, 4096 tok); decode GB/s %HBM"
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
@@ -282,7 +285,7 @@ def main():
               "forward_readme_fp32")
         extras["forward_readme_fp32"]["frac_of_peak"] = round(extras["forward_readme_fp32"]["tflops"] / 157.3, 4)
 
-    line = dict(metric="experts_fwd_tflops", value=round(value, 2), unit="TFLOP/s", n_gpus=1, steps=args.steps,
+    line = dict(metric=METRIC, value=round(value, 2), unit="TFLOP/s", n_gpus=1, steps=args.steps,
                 warmup=args.warmup, spinup_ms=args.spinup_ms, ms_per_step=round(ms_per_step, 4), higher_is_better=True, scaling="weak",
                 vs_baseline=None, dtype="bf16", data="synthetic",
                 config=dict(workload="gptoss20b: T=4096 H=I=2880 E=32 top-4 bf16, clamped SwiGLU, capacity=T",
