@@ -66,6 +66,20 @@ def test_backward_capacity_16bit(gpu, dtype, capacity):
     assert torch.all(torch.gather(d_routing, 1, d["router_indices"])[dropped] == 0)
 
 
+@pytest.mark.parametrize("H,I", [(512, 256), (640, 320), (768, 384), (896, 192), (384, 448), (128, 128)])
+def test_backward_contraction_lengths_16bit(gpu, H, I):
+    """The input-gradient GEMMs contract over H (down) and 2I (gate_up): 2 to 14 slab pairs of 64, which covers the
+    shortest contraction the pipelined loop takes (4 pairs), odd and even pair counts (the three pair buffers of the
+    [n][k] weights rotate) and the short path below 4 pairs.  Rows per expert above 256, so that full tiles run."""
+    dtype = torch.bfloat16
+    T, E, K = 640, 2, 1
+    d = make_inputs(T, H, I, E, K, dtype, seed=H + I, w_std=0.05, bias_std=0.1)
+    gy = torch.randn(T, H, generator=torch.Generator().manual_seed(7)).to(dtype)
+    grads = run_bwd(d, gy, T, gpu)
+    want = O.experts_backward(gy, *args(d), T, compute_dtype=torch.float32)
+    check(grads, want, dtype, "contraction H=%d I=%d" % (H, I))
+
+
 @pytest.mark.parametrize("slot_weights", [False, True])
 def test_backward_capacity_and_layouts(gpu, slot_weights):
     dtype = torch.float32

@@ -5,17 +5,23 @@
 //
 //  * Global -> LDS copies are `global_load_lds_dwordx4`: every lane names its own 16-byte source and
 //    the 64 lanes of a wave fill 1 KB of LDS in lane order.  The contraction is cut into slabs of
-//    32; four slab buffers (4 x 32 KB) rotate, and a slab is requested four slabs (about 3000 MFMA
-//    cycles) before it is consumed, which covers HBM latency with one wave per SIMD.
-//  * An operand whose rows are k-contiguous in memory ([row][k]) keeps that layout in LDS
-//    (64 bytes per row) and is read with one 16-byte ds_read per MFMA operand.
+//    32; the forward's weight slabs rotate through four buffers of 16 KB and are requested three to four
+//    slabs (about 3000 MFMA cycles) before they are consumed, which covers HBM latency with one wave
+//    per SIMD; the activation rows rotate through two buffers of a slab pair (32 KB) each.
+//  * An operand whose rows are k-contiguous in memory ([row][k]) keeps that layout in LDS and is read
+//    with one 16-byte ds_read per MFMA operand.  Such operands are copied two slabs at a time (128
+//    bytes of a row per copy), so that every request to L2 is a whole cache line: with 64-byte pieces
+//    the same kernel makes 1.5 times the L2 requests and runs 10-15 % slower.
+//  * [n][k] weights (the input-gradient products) are such an operand too: their B ring is three slab
+//    pairs (160 KB of LDS with the A ring), the copies are spread four per wave over every k-step and
+//    only every second slab needs a wait and a workgroup barrier.
 //  * The forward weights are [k][n] in memory and stay [k][n] in LDS (512 bytes per k row);
 //    MFMA operands are read with `ds_read_b64_tr_b16`, the LDS transpose read of gfx950, which
 //    hands lane i of a 16-lane group column n0+i for 4 consecutive k.  No register transpose, no
 //    LDS store instruction, no staging registers.
 //  * LDS swizzles are applied on the global side (a lane picks which 16-byte piece it fetches), as
 //    the LDS side of an asynchronous copy is fixed to lane order:
-//        [row][k] tiles: piece c of row r sits at position c ^ ((r >> 2) & 3)
+//        [row][k] tiles: piece c (0..7, two slabs) of row r sits at position c ^ ((r >> 1) & 7)
 //        [k][n]  tiles: piece c of row k sits at position c ^ ((k & 3) << 2)
 //    so that both kinds of MFMA operand reads touch every bank once.
 //  * Software pipeline per slab (two k-steps of 16): the operands of the second k-step are read
@@ -27,7 +33,7 @@
 // The interleaved (gate, up) columns of the clamped SwiGLU (csrc/moe.cpp:164-180) end up in
 // neighbouring lanes of one accumulator tile; the epilogue swaps them with one DPP move per pair.
 //
-// Requirements: contraction length a multiple of 32, leading dimensions multiples of 8 elements.
+// Requirements: contraction length a multiple of 64, leading dimensions multiples of 8 elements.
 // Other shapes and fp32 use gemm.hip.
 #include <type_traits>
 
@@ -45,6 +51,9 @@ constexpr int kBRing = kAStages * kAStageBytes;    // byte offset of the B ring
 constexpr int kRingBytes = kBRing + kBStages * kBStageBytes;  // 128 KB
 constexpr int kStagingBytes = kBM * (kBN * 2 + 16);            // output tile staged for the row-wise store
 constexpr int kLds = kStagingBytes > kRingBytes ? kStagingBytes : kRingBytes;
+// [n][k] weights (the input-gradient products) keep B in slab pairs as well, three of them: 160 KB with the A ring
+constexpr int kBPairStages = 3, kBPairBytes = 32768;
+constexpr int kLdsNk = kBRing + kBPairStages * kBPairBytes;
 
 static_assert(kBM == kRowTile, "row tiles of the schedule must match the GEMM tile");
 
@@ -93,8 +102,8 @@ __device__ inline u32x2 lds_read_tr16(const char *p) {
 }
 
 // what one slab step of the pipeline issues besides its MFMAs
-template <bool P1A_, bool P1B_, bool P2A_, bool P2B_, bool NEXT_, int VM_> struct StepCfg {
-  static constexpr bool P1A = P1A_, P1B = P1B_, P2A = P2A_, P2B = P2B_, NEXT = NEXT_;
+template <bool P1A_, bool P1B_, bool P2A_, bool P2B_, bool NEXT_, int VM_, bool BAR_ = true> struct StepCfg {
+  static constexpr bool P1A = P1A_, P1B = P1B_, P2A = P2A_, P2B = P2B_, NEXT = NEXT_, BAR = BAR_;
   static constexpr int VM = VM_;
 };
 
@@ -104,7 +113,7 @@ struct TileInfo {
 
 template <typename T, int EPI, int NMI, bool BNK>
 __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int tid, const char *a_base,
-                                const uint32_t (&a_off)[8], const char *b_base, const uint32_t (&b_off)[4],
+                                const uint32_t (&a_off)[8], const char *b_base, const uint32_t (&b_off)[8],
                                 long long b_slab_bytes) {
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in a scalar register
@@ -158,11 +167,11 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
     int piece = (col >> 3) ^ (j4 << 2);
     b_rd[ni] = (g * 8 + j4) * 512 + (piece << 4) + (col & 7) * 2;
   }
-  // B operand of a [n][k] tile (BNK): 64-byte rows, row wn*128 + ni*32 + lane%32, piece ks*2 + lane/32 at
-  // position piece ^ ((row >> 2) & 3); one 16-byte read per operand, like A.
+  // B operand of a [n][k] tile (BNK): stored like A, in slab pairs of 128-byte rows; row wn*128 + ni*32 + lane%32,
+  // one 16-byte read per operand.
   int b_rdk[2];
 #pragma unroll
-  for (int ks = 0; ks < 2; ++ks) b_rdk[ks] = (wn * 128 + rl) * 64 + (((ks * 2 + g) ^ ((rl >> 2) & 3)) << 4);
+  for (int ks = 0; ks < 2; ++ks) b_rdk[ks] = (wn * 128 + rl) * 128 + (((ks * 2 + g) ^ ((rl >> 1) & 7)) << 4);
 
   u32x4 fa0[NACC], fa1[NACC], fb0[4], fb1[4];
   // Operand fragments of one k-step in the order the MFMAs want them: B0, A0, B1, B2, B3, A1, A2, A3.
@@ -175,10 +184,11 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
       fa[mi] = *(const u32x4 *)(sa + (a_rd[ks] ^ ((s & 1) << 6)) + mi * 8192);
     } else {
       const int ni = f == 0 ? 0 : f - 1;
-      const char *sb = lds + kBRing + (s & (kBStages - 1)) * kBStageBytes;
       if constexpr (BNK) {
-        fb[ni] = *(const u32x4 *)(sb + b_rdk[ks] + ni * 2048);
+        const char *sb = lds + kBRing + ((s >> 1) % kBPairStages) * kBPairBytes;
+        fb[ni] = *(const u32x4 *)(sb + (b_rdk[ks] ^ ((s & 1) << 6)) + ni * 4096);
       } else {
+        const char *sb = lds + kBRing + (s & (kBStages - 1)) * kBStageBytes;
         u32x2 lo = lds_read_tr16(sb + b_rd[ni] + ks * 8192);
         u32x2 hi = lds_read_tr16(sb + b_rd[ni] + ks * 8192 + 2048);
         fb[ni] = (u32x4){lo[0], lo[1], hi[0], hi[1]};
@@ -204,6 +214,15 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
     copy16_to_lds(b_base + (long long)slab * b_slab_bytes, b_off[i],
                   lds0 + kBRing + (uint32_t)(slab & (kBStages - 1)) * kBStageBytes + (uint32_t)(8 * wave + 2 * i) * 512u);
   };
+  // [n][k] weights: piece c (0..7) of B pair `pair`, rows 64*wave + 8*c + (lane >> 3) like A
+  auto copy_bp = [&](int pair, int c) {
+    copy16_to_lds(b_base + (long long)pair * (2 * b_slab_bytes), b_off[c],
+                  lds0 + kBRing + (uint32_t)(pair % kBPairStages) * kBPairBytes + (uint32_t)(64 * wave + 8 * c) * 128u);
+  };
+  auto issue_bp = [&](int pair) {
+#pragma unroll
+    for (int c = 0; c < 8; ++c) copy_bp(pair, c);
+  };
 
   // ---- pipeline -----------------------------------------------------------------------------------------
   // A slab is two k-steps with one workgroup barrier between them; after the barrier of slab t nobody reads
@@ -214,15 +233,31 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
   // which is 6, 2, 2, 6 copies per wave over the four k-steps of a slab pair.  Copies retire in order, so
   // "slab s+1 has landed" is a bound on the number of younger copies in flight at the end of the first
   // k-step of slab s: 16 for even s, 6 for odd s (2 and 0 for the last two waits).
-  issue_b(0);
-  issue_a(0);
-  if (n_slabs > 1) issue_b(1);
-  if (n_slabs > 2) { issue_b(2); issue_a(1); }
-  if (n_slabs > 3) issue_b(3);
-  // Only slab 0 (the first 12 copies) has to be there to start; the waits of the slab steps below bound the
-  // number of younger copies in flight, and that bound holds for what is left of these 32 as well.
-  if (n_slabs >= 8) asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if constexpr (BNK) {
+    // [n][k] weights, both operands in slab pairs.  After the barrier of an odd slab 2p+1 pair p is dead: A pair p+2
+    // goes into its buffer during the next two k-steps and B pair p+3 during the two after those, four copies per wave
+    // in every k-step.  Only odd slabs wait (for pair p+1, with the eight copies of B pair p+2 still in flight) and
+    // only odd slabs need the workgroup barrier.
+    issue_a(0);
+    issue_bp(0);
+    if (n_slabs > 2) { issue_a(1); issue_bp(1); }
+    if (n_slabs >= 8) {
+      asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    } else {
+      if (n_slabs > 4) issue_bp(2);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+  } else {
+    issue_b(0);
+    issue_a(0);
+    if (n_slabs > 1) issue_b(1);
+    if (n_slabs > 2) { issue_b(2); issue_a(1); }
+    if (n_slabs > 3) issue_b(3);
+    // Only slab 0 (the first 12 copies) has to be there to start; the waits of the slab steps below bound the
+    // number of younger copies in flight, and that bound holds for what is left of these 32 as well.
+    if (n_slabs >= 8) asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
   __syncthreads();
   read_frags(0, 0, fa0, fb0);
 
@@ -238,7 +273,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
     typedef decltype(cfg) C;
     __builtin_amdgcn_sched_barrier(0);
     {
-      constexpr int kA = C::P1A ? 4 : 0, kB = C::P1B ? 2 : 0, kItems = kA + kB + kFrags;
+      constexpr int kA = C::P1A ? 4 : 0, kB = C::P1B ? (BNK ? 4 : 2) : 0, kItems = kA + kB + kFrags;
 #pragma unroll
       for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
         if (j < kMma) Mma<T>::run(fa0[j >> 2], fb0[j & 3], acc[j >> 2][j & 3]);
@@ -246,7 +281,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
 #pragma unroll
           for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
             if (i < kA) copy_a(s / 2 + 1, 4 + i);
-            else if (i < kA + kB) copy_b(s + 3, 2 + i - kA);
+            else if (i < kA + kB) { if constexpr (BNK) copy_bp((s + 3) / 2, 4 + i - kA); else copy_b(s + 3, 2 + i - kA); }
             else read_frag(s, 1, i - kA - kB, fa1, fb1);
           }
         }
@@ -254,13 +289,14 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
       }
     }
     if constexpr (C::VM == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else if constexpr (C::VM == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     else if constexpr (C::VM == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
     else if constexpr (C::VM == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
     else if constexpr (C::VM == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+    if constexpr (C::BAR) __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
     {
-      constexpr int kA = C::P2A ? 4 : 0, kB = C::P2B ? 2 : 0, kItems = kA + kB + (C::NEXT ? kFrags : 0);
+      constexpr int kA = C::P2A ? 4 : 0, kB = C::P2B ? (BNK ? 4 : 2) : 0, kItems = kA + kB + (C::NEXT ? kFrags : 0);
 #pragma unroll
       for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
         if (j < kMma) Mma<T>::run(fa1[j >> 2], fb1[j & 3], acc[j >> 2][j & 3]);
@@ -268,7 +304,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
 #pragma unroll
           for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
             if (i < kA) copy_a((s + 1) / 2 + 1, i);
-            else if (i < kA + kB) copy_b(s + 4, i - kA);
+            else if (i < kA + kB) { if constexpr (BNK) copy_bp(s / 2 + 2, i - kA); else copy_b(s + 4, i - kA); }
             else read_frag(s + 1, 0, i - kA - kB, fa0, fb0);
           }
         }
@@ -283,11 +319,26 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (odd && s + 3 < n_slabs) issue_a((s + 1) / 2 + 1);
-    if (s + kBStages < n_slabs) issue_b(s + kBStages);
+    if constexpr (!BNK) {
+      if (s + kBStages < n_slabs) issue_b(s + kBStages);  // ([n][k]: at most three B pairs, all requested up front)
+    }
     if (s + 1 < n_slabs) read_frags(s + 1, 0, fa0, fb0);
     mma(fa1, fb1);
   };
-  if (n_slabs >= 8) {
+  if (BNK && n_slabs >= 8) {
+    slab_step(0, StepCfg<false, false, false, true, true, -1, false>());
+    slab_step(1, StepCfg<false, true, true, false, true, 8>());
+    int s = 2;
+    for (; s + 5 < n_slabs; s += 2) {  // steady state: pair s/2 is consumed, A pair s/2 + 1 and B pair s/2 + 2 arrive
+      slab_step(s, StepCfg<true, false, false, true, true, -1, false>());
+      slab_step(s + 1, StepCfg<false, true, true, false, true, 8>());
+    }
+    // the last two pairs (s = n_slabs - 4)
+    slab_step(s, StepCfg<true, false, false, false, true, -1, false>());
+    slab_step(s + 1, StepCfg<false, false, false, false, true, 0>());
+    slab_step(s + 2, StepCfg<false, false, false, false, true, -1, false>());
+    slab_step(s + 3, StepCfg<false, false, false, false, false, -1, false>());
+  } else if (n_slabs >= 8) {
     // copies of the (first, second) k-step: A half, B half; whether slab s+1 is read; the vmcnt bound (-1: no wait)
     slab_step(0, StepCfg<false, false, false, true, true, 16>());
     slab_step(1, StepCfg<false, true, true, true, true, 6>());
@@ -458,16 +509,17 @@ __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
   const char *a_base = (const char *)((const T *)args.A + (GATHER ? 0ll : (long long)ti.row0 * args.lda));
 
   const long long b_ld_bytes = (long long)args.ldb * (long long)sizeof(T);
-  uint32_t b_off[4];
+  uint32_t b_off[8];
   const char *b_base;
   long long b_slab_bytes;
   if constexpr (BNK) {
-    // B is [n][k] (k-contiguous rows, one per output column): rows 64*wave + 16*i + (lane >> 2), 64 bytes of each
-    // per slab; LDS position lane & 3 holds piece pos ^ ((row >> 2) & 3)
+    // B is [n][k] (k-contiguous rows, one per output column), copied like A: rows 64*wave + 8*i + (lane >> 3), 128
+    // bytes (two slabs) of each per copy, so that every request is a whole cache line; LDS position lane & 7 holds
+    // piece pos ^ ((row >> 1) & 7)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      int row = 64 * wave + 16 * i + (lane >> 2);
-      int piece = (lane & 3) ^ ((row >> 2) & 3);
+    for (int i = 0; i < 8; ++i) {
+      int row = 64 * wave + 8 * i + (lane >> 3);
+      int piece = (lane & 7) ^ ((row >> 1) & 7);
       int r = min(row, args.Nd - 1 - ti.n0);  // columns past the end re-read the last one; never stored
       b_off[i] = (uint32_t)(r * b_ld_bytes + piece * 16);
     }
@@ -482,6 +534,7 @@ __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
       int col = ti.n0 + piece * 8;
       if (col >= args.Nd) col = ti.n0;  // columns past the end re-read valid ones; never stored
       b_off[i] = (uint32_t)(k * b_ld_bytes + (long long)(col - ti.n0) * (long long)sizeof(T));
+      b_off[4 + i] = 0;
     }
     b_base = (const char *)((const T *)args.B + (long long)ti.expert * args.b_expert_stride + ti.n0);
     b_slab_bytes = kBK * b_ld_bytes;
@@ -501,11 +554,12 @@ __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
 template <typename T, int EPI, bool GATHER, bool BNK>
 static int launch(const Args &args, int max_row_tiles, hipStream_t stream) {
   auto kernel = gemm_async_kernel<T, EPI, GATHER, BNK>;
+  constexpr int lds_bytes = BNK ? (kLdsNk > kLds ? kLdsNk : kLds) : kLds;
   static bool attr_done = false;  // benign race: the attribute call is idempotent
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(MaxDynamicSharedMemorySize=%d): %s", kLds, hipGetErrorString(e));
+      set_error("hipFuncSetAttribute(MaxDynamicSharedMemorySize=%d): %s", lds_bytes, hipGetErrorString(e));
       return (int)e;
     }
     attr_done = true;
@@ -513,7 +567,7 @@ static int launch(const Args &args, int max_row_tiles, hipStream_t stream) {
   long long total = (long long)max_row_tiles * args.n_col_tiles;
   if (total <= 0) return 0;
   total = (total + kXcds - 1) / kXcds * kXcds;
-  hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(kThreads), kLds, stream, args);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(kThreads), lds_bytes, stream, args);
   return check_launch("gemm_async_kernel");
 }
 
