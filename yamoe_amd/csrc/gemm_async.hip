@@ -798,8 +798,11 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
     const int c = tid % chunks;
     if (n0 + c * 8 < args.Nd) {
       T *p = (T *)args.C + ((long long)expert * args.Md + m0) * args.Nd + n0 + c * 8;
-      for (int r = tid / chunks; r < rows_m; r += rows_per_pass)
-        *(u32x4 *)(p + (long long)r * args.Nd) = *(const u32x4 *)(lds + r * stride + c * 16);
+      for (int r = tid / chunks; r < rows_m; r += rows_per_pass) {
+        // streaming stores: 1.6 GB of gradients per backward pass that nobody reads back soon would otherwise push the
+        // operand tiles out of L2
+        __builtin_nontemporal_store(*(const u32x4 *)(lds + r * stride + c * 16), (u32x4 *)(p + (long long)r * args.Nd));
+      }
     }
   }
 }
