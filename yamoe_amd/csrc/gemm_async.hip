@@ -30,8 +30,9 @@
 //    s+1 are read, and the MFMAs of the second k-step run.  All LDS and HBM latency sits behind
 //    MFMAs; only the barrier itself is exposed.
 //
-// The interleaved (gate, up) columns of the clamped SwiGLU (csrc/moe.cpp:164-180) end up in
-// neighbouring lanes of one accumulator tile; the epilogue swaps them with one DPP move per pair.
+// The MFMAs take the weights as their first operand, so that a lane's accumulators are one output row
+// and runs of four consecutive columns: the interleaved (gate, up) columns of the clamped SwiGLU
+// (csrc/moe.cpp:164-180) meet in one lane, and the staging stores are 4 or 8 bytes wide.
 //
 // Requirements: contraction length a multiple of 64, leading dimensions multiples of 8 elements.
 // Other shapes and fp32 use gemm.hip.
@@ -50,7 +51,8 @@ constexpr int kBStages = 4, kBStageBytes = 16384;  // B ring: single slabs (32 k
 constexpr int kBRing = kAStages * kAStageBytes;    // byte offset of the B ring
 constexpr int kRingBytes = kBRing + kBStages * kBStageBytes;  // 128 KB
 constexpr int kStagingBytes = kBM * (kBN * 2 + 16);            // output tile staged for the row-wise store
-constexpr int kLds = kStagingBytes > kRingBytes ? kStagingBytes : kRingBytes;
+constexpr int kBiasOff = kStagingBytes > kRingBytes ? kStagingBytes : kRingBytes;  // the tile's 256 bias values
+constexpr int kLds = kBiasOff + kBN * 2;
 // [n][k] weights (the input-gradient products) keep B in slab pairs as well, three of them: 160 KB with the A ring
 constexpr int kBPairStages = 3, kBPairBytes = 32768;
 constexpr int kLdsNk = kBRing + kBPairStages * kBPairBytes;
@@ -89,6 +91,20 @@ __device__ inline void copy16_to_lds(const void *uniform_base, uint32_t lane_byt
                :
                : "v"(lane_byte_off), "s"(uniform_base), "s"(lds_base)
                : "memory");
+}
+
+// two fp32 values rounded to T, packed low / high
+template <typename T> __device__ inline uint32_t pack2(float lo, float hi) {
+  typedef T T2 __attribute__((ext_vector_type(2)));
+  T2 v = {ElemTraits<T>::from_f32(lo), ElemTraits<T>::from_f32(hi)};
+  return __builtin_bit_cast(uint32_t, v);
+}
+// four consecutive elements of T (8-byte aligned) as fp32
+template <typename T> __device__ inline void load4_f32(const T *p, float (&out)[4]) {
+  typedef T T4 __attribute__((ext_vector_type(4)));
+  T4 v = *(const T4 *)p;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) out[i] = ElemTraits<T>::to_f32(v[i]);
 }
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -131,6 +147,13 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
       for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
 
   const int n_slabs = args.Kd / kBK;  // even: the contraction length is a multiple of 64
+
+  // The tile's bias values, one per thread, requested before anything else: they are the oldest entry of the memory
+  // queue, so the first wait of the pipeline covers them, and the epilogue finds them in a register instead of
+  // paying a memory latency per column block.  ([n][k] weights are the input-gradient products: no bias.)
+  const bool has_bias = !BNK && args.bias != nullptr;
+  T bias_reg = ElemTraits<T>::from_f32(0.0f);
+  if (has_bias) bias_reg = ((const T *)args.bias)[(long long)ti.expert * args.Nd + min(ti.n0 + tid, args.Nd - 1)];
 
   // ---- copy issue ----------------------------------------------------------------------------------
   // A pair p (slabs 2p, 2p+1): this wave fills rows 64*wave + 8*i + (lane >> 3), 128 bytes each.
@@ -203,7 +226,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
 #pragma unroll
     for (int mi = 0; mi < NMI; ++mi)
 #pragma unroll
-      for (int ni = 0; ni < 4; ++ni) Mma<T>::run(fa[mi], fb[ni], acc[mi][ni]);
+      for (int ni = 0; ni < 4; ++ni) Mma<T>::run(fb[ni], fa[mi], acc[mi][ni]);
   };
   // One 16-byte-per-lane copy: piece c (0..7) of A pair `pair`, or piece i (0..3) of B slab `slab`.
   auto copy_a = [&](int pair, int c) {
@@ -276,7 +299,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
       constexpr int kA = C::P1A ? 4 : 0, kB = C::P1B ? (BNK ? 4 : 2) : 0, kItems = kA + kB + kFrags;
 #pragma unroll
       for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
-        if (j < kMma) Mma<T>::run(fa0[j >> 2], fb0[j & 3], acc[j >> 2][j & 3]);
+        if (j < kMma) Mma<T>::run(fb0[j & 3], fa0[j >> 2], acc[j >> 2][j & 3]);
         if (j < kSlots) {
 #pragma unroll
           for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
@@ -299,7 +322,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
       constexpr int kA = C::P2A ? 4 : 0, kB = C::P2B ? (BNK ? 4 : 2) : 0, kItems = kA + kB + (C::NEXT ? kFrags : 0);
 #pragma unroll
       for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
-        if (j < kMma) Mma<T>::run(fa1[j >> 2], fb1[j & 3], acc[j >> 2][j & 3]);
+        if (j < kMma) Mma<T>::run(fb1[j & 3], fa1[j >> 2], acc[j >> 2][j & 3]);
         if (j < kSlots) {
 #pragma unroll
           for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
@@ -365,13 +388,14 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
   // The output tile is staged in LDS (the slab ring is dead by now) as [row][column] and then written
   // out row by row with 16 bytes per lane, so that a wave stores whole 512-byte (or 256-byte) row
   // segments instead of 2 bytes per lane.
-  // acc[mi][ni][v]: tile row (mi*2+wm)*32 + 8*(v/4) + 4*(lane/32) + v%4, tile column wn*128 + ni*32 + lane%32
-  const int rsub = g * 4;
-  const int expert = ti.expert, rows_valid = ti.rows_valid, n0 = ti.n0;
+  // The MFMAs run with the operands exchanged (weights as the A operand), so a lane holds one output row and four
+  // consecutive columns per register quad:
+  // acc[mi][ni][v]: tile row (mi*2+wm)*32 + lane%32, tile column wn*128 + ni*32 + 8*(v/4) + 4*(lane/32) + v%4
+  // which makes the staging stores 8 bytes wide and puts a (gate, up) pair into one lane.
+  const int rows_valid = ti.rows_valid, n0 = ti.n0;
   const long long out_row0 = ti.row0;
 
-  // rows of `width` elements, row stride width*2 + 16 bytes (the pad spreads the 2-byte stores of the
-  // two lane halves over different banks)
+  // rows of `width` elements, row stride width*2 + 16 bytes
   auto store_rows = [&](T *dst, long long ld, int col0, int width, int col_limit) {
     const int stride = width * 2 + 16;
     const int chunks = width >> 3, rows_per_pass = kThreads / chunks;
@@ -381,28 +405,37 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
     for (int r = tid / chunks; r < rows_valid; r += rows_per_pass)
       *(u32x4 *)(p + (long long)r * ld) = *(const u32x4 *)(lds + r * stride + c * 16);
   };
+  // the bias of this lane's 16 columns of column block ni, from the copy in LDS
+  auto load_bias = [&](int ni, float (&b)[16]) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      float t[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (has_bias) load4_f32((const T *)(lds + kBiasOff) + wn * 128 + ni * 32 + 8 * q + 4 * g, t);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) b[4 * q + i] = t[i];
+    }
+  };
   // natural column order: value = acc + bias[column]   (the plain product, or the pre-activations)
   auto stage_biased = [&]() {
     constexpr int stride = kBN * 2 + 16;
-    // one address per lane; everything else is a compile-time offset (two bases: the offset field holds 16 bits)
-    char *lp0 = lds + (wm * 32 + rsub) * stride + (wn * 128 + rl) * 2;
-    char *lp1 = lp0 + 128 * stride;
+    char *lp = lds + (wm * 32 + rl) * stride + (wn * 128 + 4 * g) * 2;  // one address per lane, the rest are constants
 #pragma unroll
     for (int ni = 0; ni < 4; ++ni) {
-      int lc = wn * 128 + ni * 32 + rl;
-      float bias = 0.0f;
-      if (args.bias != nullptr && n0 + lc < args.Nd)
-        bias = ElemTraits<T>::to_f32(((const T *)args.bias)[(long long)expert * args.Nd + n0 + lc]);
+      float b[16];
+      load_bias(ni, b);
 #pragma unroll
       for (int mi = 0; mi < NMI; ++mi)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          char *q = (mi < 2 ? lp0 : lp1) + ((mi & 1) * 64 + 8 * (v >> 2) + (v & 3)) * stride + ni * 64;
-          *(T *)q = ElemTraits<T>::from_f32(acc[mi][ni][v] + bias);
+        for (int q = 0; q < 4; ++q) {
+          const f32x16 &a = acc[mi][ni];
+          u32x2 v = {pack2<T>(a[4 * q] + b[4 * q], a[4 * q + 1] + b[4 * q + 1]),
+                     pack2<T>(a[4 * q + 2] + b[4 * q + 2], a[4 * q + 3] + b[4 * q + 3])};
+          *(u32x2 *)(lp + mi * 64 * stride + (ni * 32 + 8 * q) * 2) = v;
         }
     }
   };
 
+  if (has_bias) *(T *)(lds + kBiasOff + tid * 2) = bias_reg;  // (outside the ring and the staging area)
   __syncthreads();  // every wave has finished reading the slab ring
   if constexpr (EPI == EPI_STORE) {
     stage_biased();
@@ -415,33 +448,22 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
       store_rows((T *)args.C2, args.Nd, n0, kBN, args.Nd);
       __syncthreads();
     }
-    // Even lanes hold gate columns, odd lanes the matching up columns.  For each pair of accumulator
-    // rows (v, v+1) the even lane finishes row v and the odd lane row v+1 after one DPP swap.
+    // A register quad holds (gate, up, gate, up) of two neighbouring activations of one row.
     constexpr int stride = (kBN / 2) * 2 + 16;
-    const bool odd = lane & 1;
-    // tile row (mi*2+wm)*32 + 8*(v/4) + rsub + v%4 with v = 2u + odd; activation column (wn*128 + ni*32 + rl) / 2
-    char *lp = lds + (wm * 32 + rsub + (odd ? 1 : 0)) * stride + wn * 128 + (rl & ~1);
+    char *lp = lds + (wm * 32 + rl) * stride + (wn * 64 + 2 * g) * 2;
 #pragma unroll
     for (int ni = 0; ni < 4; ++ni) {
-      int lc = wn * 128 + ni * 32 + (rl & ~1);  // tile column of the gate of this lane's pair
-      float bg = 0.0f, bu = 0.0f;
-      if (args.bias != nullptr && n0 + lc + 1 < args.Nd) {
-        const T *bp = (const T *)args.bias + (long long)expert * args.Nd + n0 + lc;
-        bg = ElemTraits<T>::to_f32(bp[0]);
-        bu = ElemTraits<T>::to_f32(bp[1]);
-      }
+      float b[16];
+      load_bias(ni, b);
 #pragma unroll
-      for (int mi = 0; mi < NMI; ++mi) {
+      for (int mi = 0; mi < NMI; ++mi)
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          float xe = acc[mi][ni][2 * u], xo = acc[mi][ni][2 * u + 1];
-          float send = odd ? xe : xo;
-          float recv = __builtin_bit_cast(
-              float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, send), 0xB1 /* quad_perm [1,0,3,2] */, 0xF, 0xF, true));
-          float G = (odd ? recv : xe) + bg, U = (odd ? xo : recv) + bu;
-          *(T *)(lp + (mi * 64 + 8 * (u >> 1) + 2 * (u & 1)) * stride + ni * 32) = ElemTraits<T>::from_f32(glu_forward(G, U));
+        for (int q = 0; q < 4; ++q) {
+          const f32x16 &a = acc[mi][ni];
+          float h0 = glu_forward(a[4 * q] + b[4 * q], a[4 * q + 1] + b[4 * q + 1]);
+          float h1 = glu_forward(a[4 * q + 2] + b[4 * q + 2], a[4 * q + 3] + b[4 * q + 3]);
+          *(uint32_t *)(lp + mi * 64 * stride + (ni * 16 + 4 * q) * 2) = pack2<T>(h0, h1);
         }
-      }
     }
     __syncthreads();
     store_rows((T *)args.C, args.ldc, n0 >> 1, kBN / 2, args.Nd >> 1);
@@ -723,7 +745,7 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
       constexpr int kC = C::P1 ? 3 : 0, kItems = kC + kFrags;
 #pragma unroll
       for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
-        if (j < kMma) Mma<T>::run(fa0[j >> 2], fb0[j & 3], acc[j >> 2][j & 3]);
+        if (j < kMma) Mma<T>::run(fb0[j & 3], fa0[j >> 2], acc[j >> 2][j & 3]);
         if (j < kSlots) {
 #pragma unroll
           for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
@@ -743,7 +765,7 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
       constexpr int kC = C::P2 ? 3 : 0, kItems = kC + (C::NEXT ? kFrags : 0);
 #pragma unroll
       for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
-        if (j < kMma) Mma<T>::run(fa1[j >> 2], fb1[j & 3], acc[j >> 2][j & 3]);
+        if (j < kMma) Mma<T>::run(fb1[j & 3], fa1[j >> 2], acc[j >> 2][j & 3]);
         if (j < kSlots) {
 #pragma unroll
           for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
@@ -767,30 +789,34 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
     for (int s = 0; s < n_slabs; ++s) {
       if (kFrags > 0) read_frags(s, 1, fa1, fb1);
 #pragma unroll
-      for (int j = 0; j < kMma; ++j) Mma<T>::run(fa0[j >> 2], fb0[j & 3], acc[j >> 2][j & 3]);
+      for (int j = 0; j < kMma; ++j) Mma<T>::run(fb0[j & 3], fa0[j >> 2], acc[j >> 2][j & 3]);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       if (s + 1 < n_slabs && (s + 2) * kBK > rows) zero_tail(s + 1);
       __syncthreads();
       if (s + kSmallStages < n_slabs) copy_slab(s + kSmallStages);
       if (s + 1 < n_slabs) read_frags(s + 1, 0, fa0, fb0);
 #pragma unroll
-      for (int j = 0; j < kMma; ++j) Mma<T>::run(fa1[j >> 2], fb1[j & 3], acc[j >> 2][j & 3]);
+      for (int j = 0; j < kMma; ++j) Mma<T>::run(fb1[j & 3], fa1[j >> 2], acc[j >> 2][j & 3]);
     }
   }
 
   // epilogue: stage the tile in LDS, store whole row segments
   constexpr int stride = kBN * 2 + 16;
-  const int rsub = g * 4;
+  // (operands exchanged in the MFMAs, as in the forward kernel) acc[mi][ni][v]: tile row (mi*2+wm)*32 + lane%32,
+  // tile column wn*128 + ni*32 + 8*(v/4) + 4*(lane/32) + v%4
   __syncthreads();
   {
-    char *lp0 = lds + (wm * 32 + rsub) * stride + (wn * 128 + rl) * 2;
+    char *lp = lds + (wm * 32 + rl) * stride + (wn * 128 + 4 * g) * 2;
 #pragma unroll
     for (int ni = 0; ni < 4; ++ni)
 #pragma unroll
       for (int mi = 0; mi < NMI; ++mi)
 #pragma unroll
-        for (int v = 0; v < 16; ++v)
-          *(T *)(lp0 + (mi * 64 + 8 * (v >> 2) + (v & 3)) * stride + ni * 64) = ElemTraits<T>::from_f32(acc[mi][ni][v]);
+        for (int q = 0; q < 4; ++q) {
+          const f32x16 &a = acc[mi][ni];
+          u32x2 v = {pack2<T>(a[4 * q], a[4 * q + 1]), pack2<T>(a[4 * q + 2], a[4 * q + 3])};
+          *(u32x2 *)(lp + mi * 64 * stride + (ni * 32 + 8 * q) * 2) = v;
+        }
   }
   __syncthreads();
   {
