@@ -285,6 +285,18 @@ def main():
               "forward_readme_fp32")
         extras["forward_readme_fp32"]["frac_of_peak"] = round(extras["forward_readme_fp32"]["tflops"] / 157.3, 4)
 
+        del dr, ar
+        torch.cuda.empty_cache()
+        # For scale: the vendor library's dense GEMM (torch.matmul) on the same flop counts and operand layouts as the
+        # two forward GEMMs: [T*K, H] x [H, 2I] and [T*K, I] x [I, H], one matrix instead of 32 experts, no bias, no GLU.
+        gl = torch.Generator(device=dev).manual_seed(7)
+        xa = torch.randn(T * K, H, device=dev, generator=gl).to(torch.bfloat16)
+        for label, n_out in (("library_dense_gemm_gate_up_shape", 2 * I), ("library_dense_gemm_down_shape", H)):
+            wb = (torch.randn(H, n_out, device=dev, generator=gl) * 0.02).to(torch.bfloat16)
+            timed(lambda: torch.matmul(xa, wb), 2 * T * K * H * n_out, label)
+            del wb
+        del xa
+
     line = dict(metric=METRIC, value=round(value, 2), unit="TFLOP/s", n_gpus=1, steps=args.steps,
                 warmup=args.warmup, spinup_ms=args.spinup_ms, ms_per_step=round(ms_per_step, 4), higher_is_better=True, scaling="weak",
                 vs_baseline=None, dtype="bf16", data="synthetic",
