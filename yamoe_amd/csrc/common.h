@@ -50,6 +50,21 @@ template <> struct ElemTraits<f16_t> {
 __host__ __device__ inline size_t dtype_size(int dtype) { return dtype == YAMOE_F32 ? 4 : 2; }
 
 __host__ __device__ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// Division of 0 <= n < 2^31 by a divisor fixed per launch, as a multiply-high, an add and a shift (round-up method:
+// l = ceil(log2 d), mul = floor(2^32 * (2^l - d) / d) + 1, n / d = (mulhi(n, mul) + n) >> l; the sum stays below 2^32).
+struct FastDiv {
+  uint32_t mul, shift;
+};
+__host__ __device__ inline FastDiv make_fast_div(int d) {
+  FastDiv f;
+  uint32_t l = 0;
+  while ((1ull << l) < (unsigned long long)d) ++l;
+  f.mul = (uint32_t)(((1ull << 32) * ((1ull << l) - (unsigned long long)d)) / (unsigned long long)d + 1ull);
+  f.shift = l;
+  return f;
+}
+__device__ inline int fast_div(int n, FastDiv f) { return (int)((__umulhi((uint32_t)n, f.mul) + (uint32_t)n) >> f.shift); }
 __host__ __device__ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 // h = (clamp(U,-L,L) + 1) * g * sigmoid(alpha * g),  g = min(G, L)     (csrc/moe.cpp:164-180)

@@ -69,7 +69,8 @@ struct Args {
   void *C2;             // EPI_GLU: optional pre-activations [rows, Nd]
   const int *a_rows;    // optional gather of A rows: source row = a_rows[p] / a_div
   const int *sched;
-  int a_div, Kd, Nd, lda, ldb, ldc, n_col_tiles;
+  FastDiv a_div, n_col_div;  // divisions by the gather divisor and by n_col_tiles
+  int Kd, Nd, lda, ldb, ldc, n_col_tiles;
   long long b_expert_stride;
 };
 
@@ -508,11 +509,12 @@ __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
   TileInfo ti;
   {
     const int *tiles = args.sched + kSchedHeader;
-    int t0 = L / args.n_col_tiles;
+    int t0 = fast_div(L, args.n_col_div);
     int gfirst = tiles[8 * t0 + 3], gcount = tiles[8 * t0 + 4];
+    FastDiv by_gcount = {(uint32_t)tiles[8 * t0 + 5], (uint32_t)tiles[8 * t0 + 6]};
     int local = L - gfirst * args.n_col_tiles;
-    int col_tile = local / gcount;
-    const int *te = tiles + 8 * (gfirst + local % gcount);
+    int col_tile = fast_div(local, by_gcount);
+    const int *te = tiles + 8 * (gfirst + local - col_tile * gcount);
     ti.expert = te[0]; ti.row0 = te[1]; ti.rows_valid = te[2];
     ti.n0 = col_tile * kBN;
   }
@@ -525,7 +527,7 @@ __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
     int piece = (lane & 7) ^ ((row >> 1) & 7);
     int r = min(row, ti.rows_valid - 1);
     long long src = r;
-    if (GATHER) src = args.a_rows[ti.row0 + r] / args.a_div;
+    if (GATHER) src = fast_div(args.a_rows[ti.row0 + r], args.a_div);
     a_off[i] = (uint32_t)((src * args.lda + piece * 8) * (long long)sizeof(T));
   }
   const char *a_base = (const char *)((const T *)args.A + (GATHER ? 0ll : (long long)ti.row0 * args.lda));
@@ -871,10 +873,11 @@ int gemm_async_gate_up(const void *x, const int *sorted_idx, const void *w, cons
                        const void *sched, int N, int K, int E, int H, int I, int small_rows, hipStream_t stream) {
   async::Args a = {};
   a.A = x; a.B = w; a.bias = bias; a.C = act; a.C2 = pre;
-  a.a_rows = sorted_idx; a.a_div = K; a.sched = (const int *)sched;
+  a.a_rows = sorted_idx; a.a_div = make_fast_div(K); a.sched = (const int *)sched;
   a.Kd = H; a.Nd = 2 * I; a.lda = H; a.ldb = 2 * I; a.ldc = I;
   a.b_expert_stride = (long long)H * 2 * I;
   a.n_col_tiles = ceil_div(2 * I, async::kBN);
+  a.n_col_div = make_fast_div(a.n_col_tiles);
   return async::launch<T, async::EPI_GLU, true, false>(a, sched_grid_row_tiles(N, E, small_rows), stream);
 }
 
@@ -886,6 +889,7 @@ int gemm_async_down(const void *act, const void *w, const void *bias, void *y, c
   a.Kd = I; a.Nd = H; a.lda = I; a.ldb = H; a.ldc = H;
   a.b_expert_stride = (long long)I * H;
   a.n_col_tiles = ceil_div(H, async::kBN);
+  a.n_col_div = make_fast_div(a.n_col_tiles);
   return async::launch<T, async::EPI_STORE, false, false>(a, sched_grid_row_tiles(N, E, small_rows), stream);
 }
 
@@ -897,10 +901,11 @@ int gemm_async_dgrad(const void *g, const int *g_rows, int g_div, const void *w,
                      int E, int Kd, int Nd, hipStream_t stream) {
   async::Args a = {};
   a.A = g; a.B = w; a.bias = nullptr; a.C = out; a.sched = (const int *)sched;
-  a.a_rows = g_rows; a.a_div = g_div;
+  a.a_rows = g_rows; a.a_div = make_fast_div(g_rows != nullptr ? g_div : 1);
   a.Kd = Kd; a.Nd = Nd; a.lda = Kd; a.ldb = Kd; a.ldc = Nd;
   a.b_expert_stride = (long long)Nd * Kd;
   a.n_col_tiles = ceil_div(Nd, async::kBN);
+  a.n_col_div = make_fast_div(a.n_col_tiles);
   if (g_rows != nullptr) return async::launch<T, async::EPI_STORE, true, true>(a, sched_max_row_tiles(N, E), stream);
   return async::launch<T, async::EPI_STORE, false, true>(a, sched_max_row_tiles(N, E), stream);
 }

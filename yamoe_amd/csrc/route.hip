@@ -169,10 +169,11 @@ __device__ inline void build_schedule_wave(const int *counts, const int *offsets
     // tiles plus a remainder: tiles of one expert then advance through the contraction at the same pace
     // and the weight slabs one of them fetches are still in L2 when the others ask for them.
     int per_tile = tiles > 0 ? min(kRowTile, (ceil_div(kept, tiles) + 31) & ~31) : 0;
+    const FastDiv by_tiles = make_fast_div(tiles > 0 ? tiles : 1);  // the GEMM kernels divide by the group size
     for (int t = 0; t < tiles; ++t) {
       int *w = row_tiles + 8 * (gfirst + t);
       w[0] = e; w[1] = first + t * per_tile; w[2] = min(per_tile, kept - t * per_tile); w[3] = gfirst; w[4] = tiles;
-      w[5] = 0; w[6] = 0; w[7] = 0;
+      w[5] = (int)by_tiles.mul; w[6] = (int)by_tiles.shift; w[7] = 0;
     }
     n_small += tot_small; n_tiles += tot_tiles; n_active += tot_active; n_kept += tot_kept;
   }
