@@ -128,7 +128,11 @@ struct TileInfo {
   int expert, row0, rows_valid, n0;
 };
 
-template <typename T, int EPI, int NMI, bool BNK>
+// NMI / NNI: how many of this wave's four 32-row and four 32-column blocks of the tile hold valid rows / columns.  The
+// 32-column blocks alternate between the two wave columns (block cb belongs to wave column cb & 1), so a tile of 64
+// or 128 valid columns (the last column tile of a 2880-wide matrix) gives both wave columns a quarter or half of the
+// MFMAs instead of all of them to one.
+template <typename T, int EPI, int NMI, bool BNK, int NNI = 4>
 __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int tid, const char *a_base,
                                 const uint32_t (&a_off)[8], const char *b_base, const uint32_t (&b_off)[8],
                                 long long b_slab_bytes) {
@@ -182,35 +186,35 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
 #pragma unroll
   for (int ks = 0; ks < 2; ++ks) a_rd[ks] = (wm * 32 + rl) * 128 + (((ks * 2 + g) ^ ((rl >> 1) & 7)) << 4);
   // B operand (column block ni, k-step ks, half h): k = ks*16 + g*8 + h*4 + j, 4 columns at
-  // wn*128 + ni*32 + 16*((lane>>4)&1) + 4*q, where j = (lane&15)>>2 and q = lane&3.
+  // (ni*2+wn)*32 + 16*((lane>>4)&1) + 4*q, where j = (lane&15)>>2 and q = lane&3.
   const int j4 = (lane & 15) >> 2, q4 = lane & 3;
   int b_rd[4];
 #pragma unroll
   for (int ni = 0; ni < 4; ++ni) {
-    int col = wn * 128 + ni * 32 + 16 * ((lane >> 4) & 1) + 4 * q4;
+    int col = (ni * 2 + wn) * 32 + 16 * ((lane >> 4) & 1) + 4 * q4;
     int piece = (col >> 3) ^ (j4 << 2);
     b_rd[ni] = (g * 8 + j4) * 512 + (piece << 4) + (col & 7) * 2;
   }
-  // B operand of a [n][k] tile (BNK): stored like A, in slab pairs of 128-byte rows; row wn*128 + ni*32 + lane%32,
+  // B operand of a [n][k] tile (BNK): stored like A, in slab pairs of 128-byte rows; row (ni*2+wn)*32 + lane%32,
   // one 16-byte read per operand.
   int b_rdk[2];
 #pragma unroll
-  for (int ks = 0; ks < 2; ++ks) b_rdk[ks] = (wn * 128 + rl) * 128 + (((ks * 2 + g) ^ ((rl >> 1) & 7)) << 4);
+  for (int ks = 0; ks < 2; ++ks) b_rdk[ks] = (wn * 32 + rl) * 128 + (((ks * 2 + g) ^ ((rl >> 1) & 7)) << 4);
 
   u32x4 fa0[NACC], fa1[NACC], fb0[4], fb1[4];
   // Operand fragments of one k-step in the order the MFMAs want them: B0, A0, B1, B2, B3, A1, A2, A3.
   // Slab s sits in A pair buffer (s>>1)&1 (the odd slab of a pair 64 bytes further, by XOR) and B buffer s&3.
-  constexpr int kFrags = NMI > 0 ? 4 + NMI : 0;
+  constexpr int kFrags = NMI > 0 ? NNI + NMI : 0;
   auto read_frag = [&](int s, int ks, int f, u32x4 (&fa)[NACC], u32x4 (&fb)[4]) {
-    if (f == 1 || f >= 5) {
-      const int mi = f == 1 ? 0 : f - 4;
+    if (f == 1 || f >= 1 + NNI) {
+      const int mi = f == 1 ? 0 : f - NNI;
       const char *sa = lds + ((s >> 1) & (kAStages - 1)) * kAStageBytes;
       fa[mi] = *(const u32x4 *)(sa + (a_rd[ks] ^ ((s & 1) << 6)) + mi * 8192);
     } else {
       const int ni = f == 0 ? 0 : f - 1;
       if constexpr (BNK) {
         const char *sb = lds + kBRing + ((s >> 1) % kBPairStages) * kBPairBytes;
-        fb[ni] = *(const u32x4 *)(sb + (b_rdk[ks] ^ ((s & 1) << 6)) + ni * 4096);
+        fb[ni] = *(const u32x4 *)(sb + (b_rdk[ks] ^ ((s & 1) << 6)) + ni * 8192);
       } else {
         const char *sb = lds + kBRing + (s & (kBStages - 1)) * kBStageBytes;
         u32x2 lo = lds_read_tr16(sb + b_rd[ni] + ks * 8192);
@@ -227,7 +231,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
 #pragma unroll
     for (int mi = 0; mi < NMI; ++mi)
 #pragma unroll
-      for (int ni = 0; ni < 4; ++ni) Mma<T>::run(fb[ni], fa[mi], acc[mi][ni]);
+      for (int ni = 0; ni < NNI; ++ni) Mma<T>::run(fb[ni], fa[mi], acc[mi][ni]);
   };
   // One 16-byte-per-lane copy: piece c (0..7) of A pair `pair`, or piece i (0..3) of B slab `slab`.
   auto copy_a = [&](int pair, int c) {
@@ -291,7 +295,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
   //   first k-step:  MFMAs on set 0 + its copies + the LDS reads of the second k-step into set 1
   //   wait for slab s+1's copies; workgroup barrier
   //   second k-step: MFMAs on set 1 + its copies + the LDS reads of slab s+1's first k-step into set 0
-  constexpr int kMma = 4 * NMI;
+  constexpr int kMma = NNI * NMI;
   constexpr int kSlots = kMma > 2 ? kMma - 2 : 1;  // the last two MFMAs of a k-step carry nothing
   auto slab_step = [&](int s, auto cfg) {
     typedef decltype(cfg) C;
@@ -300,7 +304,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
       constexpr int kA = C::P1A ? 4 : 0, kB = C::P1B ? (BNK ? 4 : 2) : 0, kItems = kA + kB + kFrags;
 #pragma unroll
       for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
-        if (j < kMma) Mma<T>::run(fb0[j & 3], fa0[j >> 2], acc[j >> 2][j & 3]);
+        if (j < kMma) Mma<T>::run(fb0[j % NNI], fa0[j / NNI], acc[j / NNI][j % NNI]);
         if (j < kSlots) {
 #pragma unroll
           for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
@@ -323,7 +327,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
       constexpr int kA = C::P2A ? 4 : 0, kB = C::P2B ? (BNK ? 4 : 2) : 0, kItems = kA + kB + (C::NEXT ? kFrags : 0);
 #pragma unroll
       for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
-        if (j < kMma) Mma<T>::run(fb1[j & 3], fa1[j >> 2], acc[j >> 2][j & 3]);
+        if (j < kMma) Mma<T>::run(fb1[j % NNI], fa1[j / NNI], acc[j / NNI][j % NNI]);
         if (j < kSlots) {
 #pragma unroll
           for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
@@ -391,7 +395,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
   // segments instead of 2 bytes per lane.
   // The MFMAs run with the operands exchanged (weights as the A operand), so a lane holds one output row and four
   // consecutive columns per register quad:
-  // acc[mi][ni][v]: tile row (mi*2+wm)*32 + lane%32, tile column wn*128 + ni*32 + 8*(v/4) + 4*(lane/32) + v%4
+  // acc[mi][ni][v]: tile row (mi*2+wm)*32 + lane%32, tile column (ni*2+wn)*32 + 8*(v/4) + 4*(lane/32) + v%4
   // which makes the staging stores 8 bytes wide and puts a (gate, up) pair into one lane.
   const int rows_valid = ti.rows_valid, n0 = ti.n0;
   const long long out_row0 = ti.row0;
@@ -411,7 +415,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       float t[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-      if (has_bias) load4_f32((const T *)(lds + kBiasOff) + wn * 128 + ni * 32 + 8 * q + 4 * g, t);
+      if (has_bias) load4_f32((const T *)(lds + kBiasOff) + (ni * 2 + wn) * 32 + 8 * q + 4 * g, t);
 #pragma unroll
       for (int i = 0; i < 4; ++i) b[4 * q + i] = t[i];
     }
@@ -419,9 +423,9 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
   // natural column order: value = acc + bias[column]   (the plain product, or the pre-activations)
   auto stage_biased = [&]() {
     constexpr int stride = kBN * 2 + 16;
-    char *lp = lds + (wm * 32 + rl) * stride + (wn * 128 + 4 * g) * 2;  // one address per lane, the rest are constants
+    char *lp = lds + (wm * 32 + rl) * stride + (wn * 32 + 4 * g) * 2;  // one address per lane, the rest are constants
 #pragma unroll
-    for (int ni = 0; ni < 4; ++ni) {
+    for (int ni = 0; ni < NNI; ++ni) {
       float b[16];
       load_bias(ni, b);
 #pragma unroll
@@ -431,7 +435,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
           const f32x16 &a = acc[mi][ni];
           u32x2 v = {pack2<T>(a[4 * q] + b[4 * q], a[4 * q + 1] + b[4 * q + 1]),
                      pack2<T>(a[4 * q + 2] + b[4 * q + 2], a[4 * q + 3] + b[4 * q + 3])};
-          *(u32x2 *)(lp + mi * 64 * stride + (ni * 32 + 8 * q) * 2) = v;
+          *(u32x2 *)(lp + mi * 64 * stride + (ni * 64 + 8 * q) * 2) = v;
         }
     }
   };
@@ -451,9 +455,9 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
     }
     // A register quad holds (gate, up, gate, up) of two neighbouring activations of one row.
     constexpr int stride = (kBN / 2) * 2 + 16;
-    char *lp = lds + (wm * 32 + rl) * stride + (wn * 64 + 2 * g) * 2;
+    char *lp = lds + (wm * 32 + rl) * stride + (wn * 16 + 2 * g) * 2;
 #pragma unroll
-    for (int ni = 0; ni < 4; ++ni) {
+    for (int ni = 0; ni < NNI; ++ni) {
       float b[16];
       load_bias(ni, b);
 #pragma unroll
@@ -463,7 +467,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
           const f32x16 &a = acc[mi][ni];
           float h0 = glu_forward(a[4 * q] + b[4 * q], a[4 * q + 1] + b[4 * q + 1]);
           float h1 = glu_forward(a[4 * q + 2] + b[4 * q + 2], a[4 * q + 3] + b[4 * q + 3]);
-          *(uint32_t *)(lp + mi * 64 * stride + (ni * 16 + 4 * q) * 2) = pack2<T>(h0, h1);
+          *(uint32_t *)(lp + mi * 64 * stride + (ni * 32 + 4 * q) * 2) = pack2<T>(h0, h1);
         }
     }
     __syncthreads();
@@ -566,13 +570,25 @@ __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
 
   const int n_blocks32 = (ti.rows_valid + 31) >> 5;
   const int n_mi = (n_blocks32 - wm + 1) >> 1;
-  switch (n_mi) {
-    case 4: run_tile<T, EPI, 4, BNK>(args, ti, tid, a_base, a_off, b_base, b_off, b_slab_bytes); break;
-    case 3: run_tile<T, EPI, 3, BNK>(args, ti, tid, a_base, a_off, b_base, b_off, b_slab_bytes); break;
-    case 2: run_tile<T, EPI, 2, BNK>(args, ti, tid, a_base, a_off, b_base, b_off, b_slab_bytes); break;
-    case 1: run_tile<T, EPI, 1, BNK>(args, ti, tid, a_base, a_off, b_base, b_off, b_slab_bytes); break;
-    default: run_tile<T, EPI, 0, BNK>(args, ti, tid, a_base, a_off, b_base, b_off, b_slab_bytes); break;
+  // valid 32-column blocks of this wave column (they alternate between the two); tiles of 64 or 128 valid columns with
+  // three or four row blocks per wave have instantiations of their own, everything else computes all four blocks
+  const int wn = wave & 1;
+  const int n_blocks32_n = (min(kBN, args.Nd - ti.n0) + 31) >> 5;
+  const int n_ni = (n_blocks32_n - wn + 1) >> 1;
+#define YAMOE_RUN(NMI_, NNI_) run_tile<T, EPI, NMI_, BNK, NNI_>(args, ti, tid, a_base, a_off, b_base, b_off, b_slab_bytes)
+  if (n_ni <= 2 && n_mi >= 3) {
+    if (n_ni <= 1) { if (n_mi == 4) YAMOE_RUN(4, 1); else YAMOE_RUN(3, 1); }
+    else { if (n_mi == 4) YAMOE_RUN(4, 2); else YAMOE_RUN(3, 2); }
+    return;
   }
+  switch (n_mi) {
+    case 4: YAMOE_RUN(4, 4); break;
+    case 3: YAMOE_RUN(3, 4); break;
+    case 2: YAMOE_RUN(2, 4); break;
+    case 1: YAMOE_RUN(1, 4); break;
+    default: YAMOE_RUN(0, 4); break;
+  }
+#undef YAMOE_RUN
 }
 
 template <typename T, int EPI, bool GATHER, bool BNK>
