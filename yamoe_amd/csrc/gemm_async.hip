@@ -118,6 +118,8 @@ __device__ inline u32x2 lds_read_tr16(const char *p) {
   return __builtin_bit_cast(u32x2, v);
 }
 
+template <int N> __device__ inline void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+
 // what one slab step of the pipeline issues besides its MFMAs
 template <bool P1A_, bool P1B_, bool P2A_, bool P2B_, bool NEXT_, int VM_, bool BAR_ = true> struct StepCfg {
   static constexpr bool P1A = P1A_, P1B = P1B_, P2A = P2A_, P2B = P2B_, NEXT = NEXT_, BAR = BAR_;
@@ -132,7 +134,8 @@ struct TileInfo {
 // 32-column blocks alternate between the two wave columns (block cb belongs to wave column cb & 1), so a tile of 64
 // or 128 valid columns (the last column tile of a 2880-wide matrix) gives both wave columns a quarter or half of the
 // MFMAs instead of all of them to one.
-template <typename T, int EPI, int NMI, bool BNK, int NNI = 4>
+// NAB: how many of the tile's eight 32-row blocks are copied (the others hold no valid row).
+template <typename T, int EPI, int NMI, bool BNK, int NNI = 4, int NAB = 8>
 __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int tid, const char *a_base,
                                 const uint32_t (&a_off)[8], const char *b_base, const uint32_t (&b_off)[8],
                                 long long b_slab_bytes) {
@@ -161,13 +164,17 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
   if (has_bias) bias_reg = ((const T *)args.bias)[(long long)ti.expert * args.Nd + min(ti.n0 + tid, args.Nd - 1)];
 
   // ---- copy issue ----------------------------------------------------------------------------------
-  // A pair p (slabs 2p, 2p+1): this wave fills rows 64*wave + 8*i + (lane >> 3), 128 bytes each.
+  // A pair p (slabs 2p, 2p+1): copy i is the 32-row block i of the tile, this wave fills its rows 8*wave + (lane >> 3),
+  // 128 bytes each.  Blocks without valid rows (i >= n_ablk) are not copied: nobody reads them, and a tile of 192 rows,
+  // the common one, moves an eighth less through the L1 than a full one.  (The count is a template parameter: a
+  // run-time test around every copy and a run-time wait count cost more than the copies saved.)
+  constexpr int n_ablk = NAB;
   auto issue_a = [&](int pair) {
     const uint32_t stage = lds0 + (uint32_t)(pair & (kAStages - 1)) * kAStageBytes;
     const char *ab = a_base + (long long)pair * (2 * kBK * (int)sizeof(T));
 #pragma unroll
     for (int i = 0; i < 8; ++i)
-      copy16_to_lds(ab, a_off[i], stage + (uint32_t)(64 * wave + 8 * i) * 128u);
+      if (i < n_ablk) copy16_to_lds(ab, a_off[i], stage + (uint32_t)(32 * i + 8 * wave) * 128u);
   };
   // B slab: this wave fills k rows 8*wave + 2*i + (lane >> 5), 512 bytes each.
   auto issue_b = [&](int slab) {
@@ -235,8 +242,9 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
   };
   // One 16-byte-per-lane copy: piece c (0..7) of A pair `pair`, or piece i (0..3) of B slab `slab`.
   auto copy_a = [&](int pair, int c) {
-    copy16_to_lds(a_base + (long long)pair * (2 * kBK * (int)sizeof(T)), a_off[c],
-                  lds0 + (uint32_t)(pair & (kAStages - 1)) * kAStageBytes + (uint32_t)(64 * wave + 8 * c) * 128u);
+    if (c < n_ablk)
+      copy16_to_lds(a_base + (long long)pair * (2 * kBK * (int)sizeof(T)), a_off[c],
+                    lds0 + (uint32_t)(pair & (kAStages - 1)) * kAStageBytes + (uint32_t)(32 * c + 8 * wave) * 128u);
   };
   auto copy_b = [&](int slab, int i) {
     copy16_to_lds(b_base + (long long)slab * b_slab_bytes, b_off[i],
@@ -260,7 +268,8 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
   //   first k-step of slab t:   (t even) second half of A pair t/2 + 1;    second half of B slab t + 3
   // which is 6, 2, 2, 6 copies per wave over the four k-steps of a slab pair.  Copies retire in order, so
   // "slab s+1 has landed" is a bound on the number of younger copies in flight at the end of the first
-  // k-step of slab s: 16 for even s, 6 for odd s (2 and 0 for the last two waits).
+  // k-step of slab s: for even s two B slabs and one A pair (8 + the pair's copies, 16 for a full tile), for odd s 6
+  // (2 and 0 for the last two waits).
   if constexpr (BNK) {
     // [n][k] weights, both operands in slab pairs.  After the barrier of an odd slab 2p+1 pair p is dead: A pair p+2
     // goes into its buffer during the next two k-steps and B pair p+3 during the two after those, four copies per wave
@@ -270,7 +279,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
     issue_bp(0);
     if (n_slabs > 2) { issue_a(1); issue_bp(1); }
     if (n_slabs >= 8) {
-      asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+      wait_vmcnt<8 + NAB>();  // pair 0 is there when only A pair 1 (n_ablk copies) and B pair 1 (8) are in flight
     } else {
       if (n_slabs > 4) issue_bp(2);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -281,9 +290,9 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
     if (n_slabs > 1) issue_b(1);
     if (n_slabs > 2) { issue_b(2); issue_a(1); }
     if (n_slabs > 3) issue_b(3);
-    // Only slab 0 (the first 12 copies) has to be there to start; the waits of the slab steps below bound the
+    // Only slab 0 (the first 4 + n_ablk copies) has to be there to start; the waits of the slab steps below bound the
     // number of younger copies in flight, and that bound holds for what is left of these 32 as well.
-    if (n_slabs >= 8) asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
+    if (n_slabs >= 8) wait_vmcnt<12 + NAB>();  // B1, B2, B3 (12) and A pair 1 (n_ablk)
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
   __syncthreads();
@@ -316,7 +325,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    if constexpr (C::VM == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    if constexpr (C::VM == 16) wait_vmcnt<8 + NAB>();  // two B slabs (8) and one A pair (n_ablk copies) may be in flight
     else if constexpr (C::VM == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     else if constexpr (C::VM == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
     else if constexpr (C::VM == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
@@ -523,11 +532,11 @@ __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
     ti.n0 = col_tile * kBN;
   }
 
-  // A copies: rows 64*wave + 8*i + (lane >> 3); LDS position lane & 7 holds piece pos ^ ((row >> 1) & 7)
+  // A copies: copy i fetches rows 32*i + 8*wave + (lane >> 3); LDS position lane & 7 holds piece pos ^ ((row >> 1) & 7)
   uint32_t a_off[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    int row = 64 * wave + 8 * i + (lane >> 3);
+    int row = 32 * i + 8 * wave + (lane >> 3);
     int piece = (lane & 7) ^ ((row >> 1) & 7);
     int r = min(row, ti.rows_valid - 1);
     long long src = r;
@@ -576,11 +585,16 @@ __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
   const int n_blocks32_n = (min(kBN, args.Nd - ti.n0) + 31) >> 5;
   const int n_ni = (n_blocks32_n - wn + 1) >> 1;
 #define YAMOE_RUN(NMI_, NNI_) run_tile<T, EPI, NMI_, BNK, NNI_>(args, ti, tid, a_base, a_off, b_base, b_off, b_slab_bytes)
+#define YAMOE_RUN6(NNI_) run_tile<T, EPI, 3, BNK, NNI_, 6>(args, ti, tid, a_base, a_off, b_base, b_off, b_slab_bytes)
+  // six row blocks (161..192 rows, what an expert with a few rows more than two full tiles is cut into): both wave
+  // rows have three, and only six of the eight blocks are copied
+  const bool six = n_blocks32 == 6;
   if (n_ni <= 2 && n_mi >= 3) {
-    if (n_ni <= 1) { if (n_mi == 4) YAMOE_RUN(4, 1); else YAMOE_RUN(3, 1); }
-    else { if (n_mi == 4) YAMOE_RUN(4, 2); else YAMOE_RUN(3, 2); }
+    if (n_ni <= 1) { if (n_mi == 4) YAMOE_RUN(4, 1); else if (six) YAMOE_RUN6(1); else YAMOE_RUN(3, 1); }
+    else { if (n_mi == 4) YAMOE_RUN(4, 2); else if (six) YAMOE_RUN6(2); else YAMOE_RUN(3, 2); }
     return;
   }
+  if (six) { YAMOE_RUN6(4); return; }
   switch (n_mi) {
     case 4: YAMOE_RUN(4, 4); break;
     case 3: YAMOE_RUN(3, 4); break;
@@ -589,6 +603,7 @@ __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
     default: YAMOE_RUN(0, 4); break;
   }
 #undef YAMOE_RUN
+#undef YAMOE_RUN6
 }
 
 template <typename T, int EPI, bool GATHER, bool BNK>
