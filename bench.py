@@ -35,7 +35,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch of the gate_up GEMM on the GPT-OSS-20B workload, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this file (profiles/gemm_async_and_stream_gemm_counters.md): 713 500 KiB fetched x 2.0
 # (FETCH_SIZE reads half of a 1 GiB copy's bytes on this device) + 94 046 KiB written x 1.0.
-GATE_UP_TRAFFIC_BYTES = 1.557e9
+GATE_UP_TRAFFIC_BYTES = 1.627e9
 
 
 def spin_up(fn, ms):
