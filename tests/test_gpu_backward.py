@@ -80,6 +80,20 @@ def test_backward_contraction_lengths_16bit(gpu, H, I):
     check(grads, want, dtype, "contraction H=%d I=%d" % (H, I))
 
 
+@pytest.mark.parametrize("rows", [180, 250])
+def test_backward_partial_column_tiles_16bit(gpu, rows):
+    """As the forward test of the same name: output widths of 576 (64 columns in the last tile) for both input
+    gradients, 640 for the recomputed gate_up, on tiles of six and eight row blocks."""
+    dtype = torch.bfloat16
+    T, H, I, E, K = 2 * rows, 576, 576, 2, 1
+    d = make_inputs(T, H, I, E, K, dtype, seed=rows, w_std=0.05, bias_std=0.1)
+    d["router_indices"] = (torch.arange(T) % E).reshape(T, 1)
+    gy = torch.randn(T, H, generator=torch.Generator().manual_seed(8)).to(dtype)
+    grads = run_bwd(d, gy, T, gpu)
+    want = O.experts_backward(gy, *args(d), T, compute_dtype=torch.float32)
+    check(grads, want, dtype, "partial column tiles rows=%d" % rows)
+
+
 @pytest.mark.parametrize("slot_weights", [False, True])
 def test_backward_capacity_and_layouts(gpu, slot_weights):
     dtype = torch.float32

@@ -62,6 +62,20 @@ def test_forward_capacity_drop_and_slot_weights(gpu, dtype):
     assert torch.equal(run_op(d2, 60, gpu), base)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows", [180, 250, 100])
+def test_forward_partial_column_tiles(gpu, dtype, rows):
+    """H = 576 and 2I = 640: the last column tile of the down product has 64 valid columns, that of gate_up 128, on the
+    pipelined path (18 and 10 slabs).  180 rows per expert are six 32-row blocks (the tile form that copies six of
+    eight row blocks), 250 are eight, 100 take the general form."""
+    T, H, I, E, K = 2 * rows, 576, 320, 2, 1
+    d = make_inputs(T, H, I, E, K, dtype, seed=rows, w_std=0.05, bias_std=0.1)
+    d["router_indices"] = (torch.arange(T) % E).reshape(T, 1)
+    got = run_op(d, T, gpu)
+    want = oracle_forward(d, T)
+    assert report("partial column tiles", got, want, REL_L2_TOL[dtype]) < REL_L2_TOL[dtype]
+
+
 def test_forward_uneven_tile_costs(gpu):
     """Eight experts with 2048 rows each and 56 experts with 20 rows each: the shares of the tile list that the
     8 XCDs get are equal in cost, so the shares made of small tiles hold more tiles than the grid has workgroups
