@@ -135,10 +135,26 @@ __global__ __launch_bounds__(kRowThreads) void combine_backward_kernel(
     const T *bd = down_bias + (size_t)e * H;
     T *o = g_y_perm + (size_t)p * H;
     float dot = 0.0f;
-    for (int c = lane; c < H; c += kWave) {
-      float gv = ElemTraits<T>::to_f32(g[c]);
-      dot += gv * ElemTraits<T>::to_f32(bd[c]);
-      o[c] = ElemTraits<T>::from_f32(gv * w);
+    constexpr int V = ElemTraits<T>::kVec;
+    if (H % V == 0) {  // 16 bytes per lane (rows are 16-byte aligned then)
+      for (int c = lane; c < H / V; c += kWave) {
+        u32x4 graw = ((const u32x4 *)g)[c], braw = ((const u32x4 *)bd)[c], oraw;
+        const T *gv = (const T *)&graw, *bv = (const T *)&braw;
+        T *ov = (T *)&oraw;
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+          float x = ElemTraits<T>::to_f32(gv[j]);
+          dot += x * ElemTraits<T>::to_f32(bv[j]);
+          ov[j] = ElemTraits<T>::from_f32(x * w);
+        }
+        ((u32x4 *)o)[c] = oraw;
+      }
+    } else {
+      for (int c = lane; c < H; c += kWave) {
+        float gv = ElemTraits<T>::to_f32(g[c]);
+        dot += gv * ElemTraits<T>::to_f32(bd[c]);
+        o[c] = ElemTraits<T>::from_f32(gv * w);
+      }
     }
     for (int d = kWave / 2; d > 0; d >>= 1) dot += __shfl_xor(dot, d);
     if (lane == 0) {
