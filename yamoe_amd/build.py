@@ -24,6 +24,8 @@ HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall",
     # packed fp32 VALU forms are switched off on purpose (they have produced silent wrong results)
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the asynchronous-copy asm statements name M0 as clobbered; clang warns that M0 is a reserved register
+    "-Wno-inline-asm",
 ] + os.environ.get("YAMOE_HIPCC_EXTRA", "").split()
 
 

@@ -42,12 +42,15 @@ int gemm_gate_up(const void *, const int *, const void *, const void *, void *, 
 template <typename T>
 int gemm_down(const void *, const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);
 template <typename T>
-int gemm_dgrad(const void *, const int *, int, const void *, void *, const void *, int, int, int, int, hipStream_t);
+int gemm_dgrad(const void *, const int *, int, const void *, void *, const void *, int, int, int, int, const void *,
+               float *, hipStream_t);
 template <typename T>
 int gemm_wgrad(const void *, const void *, void *, const int *, const int *, int, int, int, int, hipStream_t);
 template <typename T>
-int glu_backward_rows(const void *, const void *, const float *, const float *, const int *, const int *, const void *,
-                      int, int, void *, void *, int, int, int, int, hipStream_t);
+int glu_backward_rows(const void *, const void *, const float *, const float *, int, const int *, const int *, void *,
+                      float *, int, int, hipStream_t);
+template <typename T>
+int launch_routing_grad(const float *, const int *, const void *, int, int, void *, int, int, int, hipStream_t);
 template <typename T>
 int stream_gate_up(const void *, const int *, const void *, const void *, void *, void *, const void *, int, int, int,
                    int, int, hipStream_t);
@@ -62,7 +65,7 @@ int gemm_async_down(const void *, const void *, const void *, void *, const void
                     hipStream_t);
 template <typename T>
 int gemm_async_dgrad(const void *, const int *, int, const void *, void *, const void *, int, int, int, int,
-                     hipStream_t);
+                     const void *, float *, hipStream_t);
 template <typename T>
 int gemm_async_wgrad(const void *, const void *, void *, const int *, const int *, int, int, int, int, hipStream_t);
 bool gemm_async_supported(int Kd, int Nd, int lda, int ldb, long long a_span_bytes);
@@ -95,15 +98,17 @@ static int tiles_down(const void *act, const void *w, const void *bias, void *y,
 }
 
 // g_rows == nullptr: g holds one row per sorted row; otherwise row p of the product reads g[g_rows[p] / g_div]
-// (g_span_bytes = size of the gathered tensor)
+// (g_span_bytes = size of the gathered tensor).  With dot_part the kernels also leave, per row, 2 * ceil(Nd / 256)
+// partial sums of <fp32 product row, dot_with row> (dot_with has the output's shape).
 template <typename T>
 static int tiles_dgrad(const void *g, const int *g_rows, int g_div, long long g_span_bytes, const void *w, void *out,
-                       const void *sched, int N, int E, int Kd, int Nd, hipStream_t stream) {
+                       const void *sched, int N, int E, int Kd, int Nd, const void *dot_with, float *dot_part,
+                       hipStream_t stream) {
   if constexpr (sizeof(T) == 2) {
     if (gemm_async_supported(Kd, Nd, Kd, Kd, g_rows ? g_span_bytes : 0))
-      return gemm_async_dgrad<T>(g, g_rows, g_div, w, out, sched, N, E, Kd, Nd, stream);
+      return gemm_async_dgrad<T>(g, g_rows, g_div, w, out, sched, N, E, Kd, Nd, dot_with, dot_part, stream);
   }
-  return gemm_dgrad<T>(g, g_rows, g_div, w, out, sched, N, E, Kd, Nd, stream);
+  return gemm_dgrad<T>(g, g_rows, g_div, w, out, sched, N, E, Kd, Nd, dot_with, dot_part, stream);
 }
 
 template <typename T>
@@ -152,6 +157,11 @@ static int check_problem(const yamoe_problem *p, const char *who) {
     set_error("%s: T*K too large", who);
     return YAMOE_E_ARG;
   }
+  // the GEMM kernels address gathered token rows with 32-bit byte offsets from the start of the tensor
+  if ((long long)p->T * p->H * (long long)dtype_size(p->dtype) >= (1ll << 32)) {
+    set_error("%s: hidden_states / grad_out of 4 GiB or more are not supported (T=%d H=%d)", who, p->T, p->H);
+    return YAMOE_E_ARG;
+  }
   return 0;
 }
 
@@ -194,7 +204,8 @@ static size_t carve_forward(const yamoe_problem *p, void *ws, ForwardBuffers *b)
 struct BackwardBuffers {
   ForwardBuffers f;
   void *x_perm, *pre, *g_y_perm, *d_act, *d_pre, *d_x_perm;
-  float *w_sorted, *dot_bias;
+  float *w_sorted, *row_dot, *dot_part;
+  int n_part;
 };
 
 static size_t carve_backward(const yamoe_problem *p, void *ws, BackwardBuffers *b) {
@@ -209,7 +220,11 @@ static size_t carve_backward(const yamoe_problem *p, void *ws, BackwardBuffers *
   b->d_act = b->f.y_perm;
   b->d_x_perm = c.take(N * p->H * es);
   b->w_sorted = (float *)c.take(N * sizeof(float));
-  b->dot_bias = (float *)c.take(N * sizeof(float));
+  b->row_dot = (float *)c.take(N * sizeof(float));
+  // 16-bit data: partial row dots of the down projection's input gradient with the activations, two per 256-column
+  // tile of I, written by that GEMM from its fp32 accumulators
+  b->n_part = es == 2 ? 2 * ceil_div(p->I, kColTile) : 0;
+  b->dot_part = b->n_part ? (float *)c.take(N * (size_t)b->n_part * sizeof(float)) : nullptr;
   // the weight-gradient kernel's copies of an expert's last, partial slab of rows run up to 32 rows past the
   // end of its operand buffers; every operand is followed by another buffer of this workspace, and this pad
   // covers the case where those are smaller than 32 rows of the widest operand
@@ -271,19 +286,21 @@ static int backward_impl(const yamoe_problem *p, const void *gy, const void *x, 
   YAMOE_TRY(tiles_gate_up<T>(x, b.f.sorted_idx, wgu, bgu, b.f.act, b.pre, b.f.schedule, N, p->K, E, H, I, 0, stream));
   // combine backward: g_y_perm = grad_out[tok] * w, and the bias part of the routing gradient
   YAMOE_TRY(launch_combine_backward<T>(gy, bd, b.f.sorted_idx, b.f.inv_pos, idx, p->idx_i64, rw, p->rw_cols, b.g_y_perm,
-                                       b.w_sorted, b.dot_bias, N, p->K, E, H, stream));
+                                       b.w_sorted, b.row_dot, N, p->K, E, H, stream));
   // down projection: bias and weight gradients from the weighted rows; the input gradient from the un-weighted
   // rows of grad_out, gathered by token (its dot with the activations is the rest of the routing gradient)
   YAMOE_TRY(launch_expert_colsum<T>(b.g_y_perm, b.f.counts, b.f.offsets, cap, d_bd, E, H, stream));
   YAMOE_TRY(tiles_dgrad<T>(gy, b.f.sorted_idx, p->K, (long long)p->T * H * (long long)es, wd, b.d_act, b.f.schedule, N, E,
-                           /*Kd=*/H, /*Nd=*/I, stream));
+                           /*Kd=*/H, /*Nd=*/I, b.f.act, b.dot_part, stream));
   YAMOE_TRY(tiles_wgrad<T>(b.f.act, b.g_y_perm, d_wd, b.f.counts, b.f.offsets, cap, E, /*Md=*/I, /*Nd=*/H, stream));
   // GLU backward (scaled by the routing weight) and the routing gradient
-  YAMOE_TRY(glu_backward_rows<T>(b.d_act, b.pre, b.w_sorted, b.dot_bias, b.f.sorted_idx, b.f.inv_pos, idx, p->idx_i64,
-                                 p->rw_cols, b.d_pre, d_rw, N, p->K, E, I, stream));
+  YAMOE_TRY(glu_backward_rows<T>(b.d_act, b.pre, b.w_sorted, b.dot_part, b.n_part, b.f.sorted_idx, b.f.inv_pos, b.d_pre,
+                                 b.row_dot, N, I, stream));
+  YAMOE_TRY(launch_routing_grad<T>(b.row_dot, b.f.inv_pos, idx, p->idx_i64, p->rw_cols, d_rw, N, p->K, E, stream));
   // gate_up projection
   YAMOE_TRY(launch_expert_colsum<T>(b.d_pre, b.f.counts, b.f.offsets, cap, d_bgu, E, 2 * I, stream));
-  YAMOE_TRY(tiles_dgrad<T>(b.d_pre, nullptr, 1, 0, wgu, b.d_x_perm, b.f.schedule, N, E, /*Kd=*/2 * I, /*Nd=*/H, stream));
+  YAMOE_TRY(tiles_dgrad<T>(b.d_pre, nullptr, 1, 0, wgu, b.d_x_perm, b.f.schedule, N, E, /*Kd=*/2 * I, /*Nd=*/H, nullptr,
+                           nullptr, stream));
   YAMOE_TRY(tiles_wgrad<T>(b.x_perm, b.d_pre, d_wgu, b.f.counts, b.f.offsets, cap, E, /*Md=*/H, /*Nd=*/2 * I, stream));
   // permute backward: d_hidden[t] = sum_k d_x_perm[inv_pos[t,k]]
   YAMOE_TRY(launch_combine<T>(b.d_x_perm, b.f.inv_pos, idx, p->idx_i64, nullptr, p->K, d_x, p->T, p->K, E, H, stream));
@@ -342,6 +359,10 @@ extern "C" int yamoe_gate_up(const void *x, const int32_t *sorted_idx, const voi
   if (N == 0) return 0;
   if (!x || !sorted_idx || !gate_up_proj || !act || !schedule || K <= 0) {
     set_error("yamoe_gate_up: null pointer or K <= 0");
+    return YAMOE_E_ARG;
+  }
+  if ((long long)(N / K) * H * (long long)dtype_size(dtype) >= (1ll << 32)) {
+    set_error("yamoe_gate_up: x of 4 GiB or more is not supported (rows gathered with 32-bit byte offsets)");
     return YAMOE_E_ARG;
   }
   YAMOE_DISPATCH(dtype, gate_up_both<T>(x, sorted_idx, gate_up_proj, gate_up_proj_bias, act, pre_act, schedule, N, K,

@@ -103,6 +103,7 @@ __device__ inline void glu_backward(float G, float U, float dh, float &dG, float
 //                       index of the expert's first row tile, number of row tiles of the expert, 0,0,0}
 //   then              small experts: 4 words each {expert, first sorted row, valid rows, 0}
 constexpr int kRowTile = 256;  // rows of one MFMA row tile
+constexpr int kColTile = 256;  // columns of one MFMA tile
 constexpr int kSchedHeader = 48;
 constexpr int kSchedCuts = 8;  // word offset of the XCD cut table
 constexpr int kXcds = 8;

@@ -39,7 +39,7 @@ constexpr int kRowBytes = 128;                 // bytes of one LDS tile row (one
 constexpr int kTileBytes = kBM * kRowBytes;    // 32 KB per operand per stage
 constexpr int kGemmLds = 4 * kTileBytes;       // A,B x 2 stages = 128 KB
 
-static_assert(kBM == kRowTile, "row tiles of the schedule must match the GEMM tile");
+static_assert(kBM == kRowTile && kBN == kColTile, "tiles of the schedule must match the GEMM tile");
 
 enum { OP_KCONTIG = 0, OP_TRANSPOSED = 1 };
 enum {
@@ -65,6 +65,10 @@ struct GemmArgs {
   long long c_expert_stride;  // elements between experts in C (PROB_WGRAD)
   int n_col_tiles, n_row_tiles_wgrad;
   int N, E, capacity;
+  // PROB_ROWS + EPI_STORE, optional: dot_part[row][2 * col_tile + wave column] = the fp32 accumulators of the row times
+  // dot_with[row][same columns] (a [rows, ldc] tensor), summed over the wave's 128 columns
+  const void *dot_with;
+  float *dot_part;
 };
 
 __device__ inline int lds_swizzle(int row) { return (row ^ (row >> 3)) & 7; }
@@ -326,6 +330,41 @@ __device__ inline void run_tile(const GemmArgs &args, const TileInfo &ti, LA &la
   const int expert = ti.expert, rows_valid = ti.rows_valid, n0 = ti.n0;
   const long long out_row0 = (PROB == PROB_WGRAD) ? ti.m0 : ti.row0;
   const bool full = rows_valid == kBM && n0 + kBN <= args.Nd;
+  if constexpr (EPI == EPI_STORE && PROB == PROB_ROWS) {
+    // Row dots of the product with a second tensor of the output's shape, from the fp32 accumulators (the routing
+    // gradient <grad_out . W_down^T, act>, csrc/experts_backward.cu:83-88): one partial sum per valid row and wave,
+    // over the wave's 128 columns of the tile.
+    if (args.dot_part != nullptr) {
+      const int n_part = 2 * args.n_col_tiles, part_col = 2 * (n0 / kBN) + wn;
+#pragma unroll
+      for (int mi = 0; mi < NMI; ++mi) {
+        float part[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int r = (mi * 2 + wm) * 32 + 8 * (v >> 2) + rsub + (v & 3);
+          const T *wp = (const T *)args.dot_with + (out_row0 + min(r, rows_valid - 1)) * args.ldc;
+          float sum = 0.0f;
+#pragma unroll
+          for (int ni = 0; ni < 4; ++ni) {
+            const int col = n0 + wn * 128 + ni * 32 + lcol;
+            if (col < args.Nd) sum += acc[mi][ni][v] * ElemTraits<T>::to_f32(wp[col]);
+          }
+          part[v] = sum;
+        }
+#pragma unroll
+        for (int d = 1; d < 32; d <<= 1)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) part[v] += __shfl_xor(part[v], d);
+        if (lcol == 0) {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int r = (mi * 2 + wm) * 32 + 8 * (v >> 2) + rsub + (v & 3);
+            if (r < rows_valid) args.dot_part[(out_row0 + r) * n_part + part_col] = part[v];
+          }
+        }
+      }
+    }
+  }
   if constexpr (EPI == EPI_STORE) {
     T *C = (T *)args.C + ((PROB == PROB_WGRAD) ? (long long)expert * args.c_expert_stride : 0);
 #pragma unroll
@@ -536,9 +575,10 @@ int gemm_down(const void *act, const void *w, const void *bias, void *y, const v
 // source row of p is g_rows[p] / g_div (rows of a [T, Kd] tensor gathered by token).
 template <typename T>
 int gemm_dgrad(const void *g, const int *g_rows, int g_div, const void *w, void *d_out, const void *sched, int N, int E,
-               int Kd, int Nd, hipStream_t stream) {
+               int Kd, int Nd, const void *dot_with, float *dot_part, hipStream_t stream) {
   GemmArgs a = {};
   a.A = g; a.B = w; a.C = d_out; a.sched = (const int *)sched;
+  a.dot_with = dot_with; a.dot_part = dot_part;
   a.a_rows = g_rows; a.a_div = g_div;
   a.Kd = Kd; a.Nd = Nd; a.lda = Kd; a.ldb = Kd; a.ldc = Nd;
   a.b_expert_stride = (long long)Nd * Kd;
@@ -569,7 +609,7 @@ int gemm_wgrad(const void *L, const void *R, void *dW, const int *counts, const 
   template int gemm_down<T>(const void *, const void *, const void *, void *, const void *, int, int, int, int,     \
                             hipStream_t);                                                                           \
   template int gemm_dgrad<T>(const void *, const int *, int, const void *, void *, const void *, int, int, int, int, \
-                             hipStream_t);                                                                          \
+                             const void *, float *, hipStream_t);                                                   \
   template int gemm_wgrad<T>(const void *, const void *, void *, const int *, const int *, int, int, int, int,      \
                              hipStream_t);
 YAMOE_INSTANTIATE_GEMM(float)

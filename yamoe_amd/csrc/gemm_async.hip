@@ -57,7 +57,7 @@ constexpr int kLds = kBiasOff + kBN * 2;
 constexpr int kBPairStages = 3, kBPairBytes = 32768;
 constexpr int kLdsNk = kBRing + kBPairStages * kBPairBytes;
 
-static_assert(kBM == kRowTile, "row tiles of the schedule must match the GEMM tile");
+static_assert(kBM == kRowTile && kBN == kColTile, "tiles of the schedule must match the GEMM tile");
 
 enum { EPI_STORE = 0, EPI_GLU = 1 };
 
@@ -72,6 +72,10 @@ struct Args {
   FastDiv a_div, n_col_div;  // divisions by the gather divisor and by n_col_tiles
   int Kd, Nd, lda, ldb, ldc, n_col_tiles;
   long long b_expert_stride;
+  // EPI_STORE with [n][k] weights, optional: dot_part[row][2 * col_tile + wave column] = the fp32 accumulators of the
+  // row times dot_with[row][same columns] (a [rows, ldc] tensor), summed over the wave's 128 columns
+  const void *dot_with;
+  float *dot_part;
 };
 
 template <typename T> struct Mma;
@@ -91,7 +95,7 @@ __device__ inline void copy16_to_lds(const void *uniform_base, uint32_t lane_byt
   asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
                :
                : "v"(lane_byte_off), "s"(uniform_base), "s"(lds_base)
-               : "memory");
+               : "memory", "m0");
 }
 
 // two fp32 values rounded to T, packed low / high
@@ -450,6 +454,35 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
   };
 
   if (has_bias) *(T *)(lds + kBiasOff + tid * 2) = bias_reg;  // (outside the ring and the staging area)
+  if constexpr (EPI == EPI_STORE && BNK) {
+    // Row dots of the product with a second tensor of the output's shape, taken from the fp32 accumulators before they
+    // are rounded (the routing gradient <grad_out . W_down^T, act>, csrc/experts_backward.cu:83-88): every wave writes
+    // one partial sum per valid row, over its 128 columns of the tile; whoever reads them adds 2 * n_col_tiles values
+    // per row in a fixed order.
+    if (args.dot_part != nullptr) {
+      const int n_part = 2 * args.n_col_tiles, part_col = 2 * (n0 / kBN) + wn;
+#pragma unroll
+      for (int mi = 0; mi < NMI; ++mi) {
+        const int r = (mi * 2 + wm) * 32 + rl;
+        const T *wp = (const T *)args.dot_with + (out_row0 + min(r, rows_valid - 1)) * args.ldc + n0 + wn * 32 + 4 * g;
+        float part = 0.0f;
+#pragma unroll
+        for (int ni = 0; ni < NNI; ++ni)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            // a run of four columns is valid or invalid as a whole (the column count is a multiple of 8)
+            if (n0 + (ni * 2 + wn) * 32 + 8 * q + 4 * g < args.Nd) {
+              float w4[4];
+              load4_f32(wp + ni * 64 + 8 * q, w4);
+#pragma unroll
+              for (int i = 0; i < 4; ++i) part += acc[mi][ni][4 * q + i] * w4[i];
+            }
+          }
+        part += __shfl_xor(part, 32);
+        if (g == 0 && r < rows_valid) args.dot_part[(out_row0 + r) * n_part + part_col] = part;
+      }
+    }
+  }
   __syncthreads();  // every wave has finished reading the slab ring
   if constexpr (EPI == EPI_STORE) {
     stage_biased();
@@ -929,9 +962,10 @@ int gemm_async_down(const void *act, const void *w, const void *bias, void *y, c
 // With g_rows the source row of sorted row p is g_rows[p] / g_div (rows of a [T, Kd] tensor gathered by token).
 template <typename T>
 int gemm_async_dgrad(const void *g, const int *g_rows, int g_div, const void *w, void *out, const void *sched, int N,
-                     int E, int Kd, int Nd, hipStream_t stream) {
+                     int E, int Kd, int Nd, const void *dot_with, float *dot_part, hipStream_t stream) {
   async::Args a = {};
   a.A = g; a.B = w; a.bias = nullptr; a.C = out; a.sched = (const int *)sched;
+  a.dot_with = dot_with; a.dot_part = dot_part;
   a.a_rows = g_rows; a.a_div = make_fast_div(g_rows != nullptr ? g_div : 1);
   a.Kd = Kd; a.Nd = Nd; a.lda = Kd; a.ldb = Kd; a.ldc = Nd;
   a.b_expert_stride = (long long)Nd * Kd;
@@ -976,7 +1010,7 @@ int gemm_async_wgrad(const void *L, const void *R, void *dW, const int *counts, 
   template int gemm_async_down<T>(const void *, const void *, const void *, void *, const void *, int, int, int, \
                                   int, int, hipStream_t);                                                             \
   template int gemm_async_dgrad<T>(const void *, const int *, int, const void *, void *, const void *, int, int, int,  \
-                                   int, hipStream_t);                                                                  \
+                                   int, const void *, float *, hipStream_t);                                           \
   template int gemm_async_wgrad<T>(const void *, const void *, void *, const int *, const int *, int, int, int, int,    \
                                    hipStream_t);
 YAMOE_INSTANTIATE_ASYNC(bf16_t)

@@ -164,17 +164,18 @@ __global__ __launch_bounds__(kRowThreads) void combine_backward_kernel(
   }
 }
 
-// GLU backward on kept rows (csrc/experts_backward.cu:285-305) plus the rest of the routing gradient:
+// GLU backward on kept rows (csrc/experts_backward.cu:285-305) plus the row's share of the routing gradient:
 //   d_act[p,:] is the input gradient of the down projection for the UN-weighted output gradient of row p,
 //   d_pre[p,:] = w_sorted[p] * glu'(pre[p,:]) applied to d_act[p,:]      (interleaved gate/up columns)
-//   d_routing[tok, expert] = <d_act[p,:], glu(pre[p,:])> + dot_bias[p]
-// One wave per row; d_routing is written once per kept (token, slot).
-template <typename T, bool I64>
+//   row_dot[p] = <d_act[p,:], glu(pre[p,:])> + row_dot[p]                (row_dot comes in holding dot_bias[p])
+// With dot_part the first term is the sum of the n_part partial sums per row that the input-gradient GEMM took
+// from its fp32 accumulators (d_act itself is rounded to the activation dtype); without it (fp32 data) the dot is
+// formed here from d_act and the recomputed activations.  One wave per row.
+template <typename T>
 __global__ __launch_bounds__(kRowThreads) void glu_backward_rows_kernel(
     const T *__restrict__ d_act, const T *__restrict__ pre, const float *__restrict__ w_sorted,
-    const float *__restrict__ dot_bias, const int *__restrict__ sorted_idx, const int *__restrict__ inv_pos,
-    const void *__restrict__ idx, int rw_cols, T *__restrict__ d_pre, T *__restrict__ d_routing, int N, int K, int E,
-    int I) {
+    const float *__restrict__ dot_part, int n_part, const int *__restrict__ sorted_idx,
+    const int *__restrict__ inv_pos, T *__restrict__ d_pre, float *__restrict__ row_dot, int N, int I) {
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = blockIdx.x * kRowWaves + threadIdx.x / kWave;
   const int n_waves = gridDim.x * kRowWaves;
@@ -201,7 +202,7 @@ __global__ __launch_bounds__(kRowThreads) void glu_backward_rows_kernel(
           float dh = ElemTraits<T>::to_f32(dv[j]);
           float dG, dU;
           glu_backward(G, U, dh * w, dG, dU);
-          dot += dh * glu_forward(G, U);
+          if (dot_part == nullptr) dot += dh * glu_forward(G, U);
           ov[2 * j] = ElemTraits<T>::from_f32(dG);
           ov[2 * j + 1] = ElemTraits<T>::from_f32(dU);
         }
@@ -213,23 +214,49 @@ __global__ __launch_bounds__(kRowThreads) void glu_backward_rows_kernel(
         float dh = ElemTraits<T>::to_f32(da[c]);
         float dG, dU;
         glu_backward(G, U, dh * w, dG, dU);
-        dot += dh * glu_forward(G, U);
+        if (dot_part == nullptr) dot += dh * glu_forward(G, U);
         dp[2 * c] = ElemTraits<T>::from_f32(dG);
         dp[2 * c + 1] = ElemTraits<T>::from_f32(dU);
       }
     }
+    if (dot_part != nullptr)
+      for (int c = lane; c < n_part; c += kWave) dot += dot_part[(size_t)p * n_part + c];
     for (int d = kWave / 2; d > 0; d >>= 1) dot += __shfl_xor(dot, d);
-    if (lane == 0) {
-      int t = flat / K, k = flat - t * K;
-      float v = dot + dot_bias[p];
-      if (rw_cols == K && rw_cols != E) {
-        d_routing[(size_t)t * K + k] = ElemTraits<T>::from_f32(v);
-      } else {
-        long long e = I64 ? ((const long long *)idx)[flat] : (long long)((const int *)idx)[flat];
-        d_routing[(size_t)t * E + e] = ElemTraits<T>::from_f32(v);
-      }
-    }
+    if (lane == 0) row_dot[p] += dot;
   }
+}
+
+// d_routing from the per-row values (csrc/experts_backward.cu:83-88, 261-271, placed once): one thread per flat slot
+// (token t, slot k).  Per-slot weights [T,K]: d_routing[t,k] = row_dot[row of the slot].  Dense weights [T,E]: the
+// first slot of the token that names expert e writes the sum over all of the token's slots that name e (a token
+// that lists an expert twice reads one weight twice), in slot order; everything else keeps the zero fill.
+template <typename T, bool I64>
+__global__ __launch_bounds__(kRowThreads) void routing_grad_kernel(const float *__restrict__ row_dot,
+                                                                   const int *__restrict__ inv_pos,
+                                                                   const void *__restrict__ idx, int rw_cols,
+                                                                   T *__restrict__ d_routing, int N, int K, int E) {
+  const int flat = blockIdx.x * kRowThreads + threadIdx.x;
+  if (flat >= N) return;
+  const int p = inv_pos[flat];
+  if (rw_cols == K && rw_cols != E) {
+    if (p >= 0) d_routing[flat] = ElemTraits<T>::from_f32(row_dot[p]);
+    return;
+  }
+  auto expert_of = [&](int f) {
+    return I64 ? ((const long long *)idx)[f] : (long long)((const int *)idx)[f];
+  };
+  const int t = flat / K, k = flat - t * K;
+  const long long e = expert_of(flat);
+  if (e < 0 || e >= E) return;
+  float sum = 0.0f;
+  bool any = false;
+  for (int k2 = 0; k2 < K; ++k2) {
+    if (expert_of(t * K + k2) != e) continue;
+    if (k2 < k) return;  // an earlier slot of the token owns this entry
+    const int p2 = inv_pos[t * K + k2];
+    if (p2 >= 0) { sum += row_dot[p2]; any = true; }
+  }
+  if (any) d_routing[(size_t)t * E + e] = ElemTraits<T>::from_f32(sum);
 }
 
 // Column sums over each expert's kept rows: out[e, c] = sum_{rows p of e} src[p, c]
@@ -341,20 +368,28 @@ int launch_combine_backward(const void *grad_out, const void *down_bias, const i
 }
 
 template <typename T>
-int glu_backward_rows(const void *d_act, const void *pre, const float *w_sorted, const float *dot_bias,
-                      const int *sorted_idx, const int *inv_pos, const void *idx, int idx_i64, int rw_cols, void *d_pre,
-                      void *d_routing, int N, int K, int E, int I, hipStream_t stream) {
+int glu_backward_rows(const void *d_act, const void *pre, const float *w_sorted, const float *dot_part, int n_part,
+                      const int *sorted_idx, const int *inv_pos, void *d_pre, float *row_dot, int N, int I,
+                      hipStream_t stream) {
   if (N == 0) return 0;
   int blocks = min(ceil_div(N, kRowWaves), 256 * 16);
-  if (idx_i64)
-    hipLaunchKernelGGL((glu_backward_rows_kernel<T, true>), dim3(blocks), dim3(kRowThreads), 0, stream, (const T *)d_act,
-                       (const T *)pre, w_sorted, dot_bias, sorted_idx, inv_pos, idx, rw_cols, (T *)d_pre, (T *)d_routing, N,
-                       K, E, I);
-  else
-    hipLaunchKernelGGL((glu_backward_rows_kernel<T, false>), dim3(blocks), dim3(kRowThreads), 0, stream, (const T *)d_act,
-                       (const T *)pre, w_sorted, dot_bias, sorted_idx, inv_pos, idx, rw_cols, (T *)d_pre, (T *)d_routing, N,
-                       K, E, I);
+  hipLaunchKernelGGL(glu_backward_rows_kernel<T>, dim3(blocks), dim3(kRowThreads), 0, stream, (const T *)d_act,
+                     (const T *)pre, w_sorted, dot_part, n_part, sorted_idx, inv_pos, (T *)d_pre, row_dot, N, I);
   return check_launch("glu_backward_rows_kernel");
+}
+
+template <typename T>
+int launch_routing_grad(const float *row_dot, const int *inv_pos, const void *idx, int idx_i64, int rw_cols,
+                        void *d_routing, int N, int K, int E, hipStream_t stream) {
+  if (N == 0) return 0;
+  int blocks = ceil_div(N, kRowThreads);
+  if (idx_i64)
+    hipLaunchKernelGGL((routing_grad_kernel<T, true>), dim3(blocks), dim3(kRowThreads), 0, stream, row_dot, inv_pos, idx,
+                       rw_cols, (T *)d_routing, N, K, E);
+  else
+    hipLaunchKernelGGL((routing_grad_kernel<T, false>), dim3(blocks), dim3(kRowThreads), 0, stream, row_dot, inv_pos, idx,
+                       rw_cols, (T *)d_routing, N, K, E);
+  return check_launch("routing_grad_kernel");
 }
 
 template <typename T>
@@ -377,9 +412,10 @@ int launch_expert_colsum(const void *src, const int *counts, const int *offsets,
   template int launch_combine_backward<T>(const void *, const void *, const int *, const int *, const void *,   \
                                           int, const void *, int, void *, float *, float *, int, int, int, int,  \
                                           hipStream_t);                                                          \
-  template int glu_backward_rows<T>(const void *, const void *, const float *, const float *, const int *,      \
-                                    const int *, const void *, int, int, void *, void *, int, int, int, int,     \
-                                    hipStream_t);                                                                \
+  template int glu_backward_rows<T>(const void *, const void *, const float *, const float *, int, const int *, \
+                                    const int *, void *, float *, int, int, hipStream_t);                        \
+  template int launch_routing_grad<T>(const float *, const int *, const void *, int, int, void *, int, int, int, \
+                                      hipStream_t);                                                              \
   template int launch_expert_colsum<T>(const void *, const int *, const int *, int, void *, int, int,  \
                                        hipStream_t);
 YAMOE_INSTANTIATE_ROWS(float)
