@@ -10,10 +10,10 @@ hide behind, so every entry is checked on its own, twice:
                        with d_act = grad_out[t] . W_down[e]^T, plus one rounding of the stored value.
   against the forward  the same dot taken in fp64 from the activations the gate_up kernel itself produced (through the
                        C ABI).  Nothing is rounded between those and the result except the fp32 accumulation and the
-                       final store, so the error allowed is 2^-12 of sqrt(sum_i (d_act_i * act_i)^2) + |<grad_out, b_down>|
+                       final store, so the error allowed is 2^-11 of sqrt(sum_i (d_act_i * act_i)^2) + |<grad_out, b_down>|
                        plus one rounding of the stored value.  A routing gradient formed from an input gradient that
                        was first rounded to the activation dtype has a typical error of 0.6 u of that root sum
-                       (u = 2^-9 for bf16), several times the bound.
+                       (u = 2^-9 for bf16): more than twice the bound on a typical entry, and every entry is checked.
 """
 import pytest
 import torch
@@ -116,7 +116,7 @@ def test_routing_grad_every_entry(gpu, dtype, T, H, I, E, K, seed, zipf, slot_we
         torch.cuda.synchronize()
         want2, _, rms2 = slot_terms(d, gy, act.cpu(), r["sorted_idx"], r["inv_pos"])
         err2 = (got - want2).abs()
-        bound2 = 2.0 ** -12 * rms2 + 2 * u * want2.abs() + 1e-30
+        bound2 = 2.0 ** -11 * rms2 + 2 * u * want2.abs() + 1e-30
         print("  vs forward activations: worst err / bound = %.3f" % float((err2 / bound2).max()), flush=True)
         assert torch.all(err2 <= bound2), (err2 / bound2).max()
 

@@ -63,6 +63,22 @@ def make_inputs(T, H, I, E, K, dtype, seed=0, w_std=0.02, bias_std=0.02, renorm=
     return out
 
 
+def device_weights(E, H, I, dtype, std, seed, device, bias_std=None):
+    """The four weight tensors drawn on `device` (N(0, std), biases N(0, bias_std), default std), expert by expert.
+    For the 128-expert shapes, where drawing 6.4 GB on the host generator takes minutes; the values depend on the
+    device's generator, so a CPU check copies them back instead of regenerating them."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    bias_std = std if bias_std is None else bias_std
+
+    def draw(shape, s):
+        t = torch.empty(shape, dtype=dtype, device=device)
+        for e in range(shape[0]):
+            t[e] = (torch.randn(shape[1:], generator=g, device=device) * s).to(dtype)
+        return t
+    return dict(gate_up_proj=draw((E, H, 2 * I), std), gate_up_proj_bias=draw((E, 2 * I), bias_std),
+                down_proj=draw((E, I, H), std), down_proj_bias=draw((E, H), bias_std))
+
+
 def make_config(name, seed=0, device="cpu", weights=True):
     c = dict(CONFIGS[name])
     return make_inputs(seed=seed, device=device, weights=weights, **c), c
