@@ -4,6 +4,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <atomic>
+
 #include "common.h"
 
 namespace yamoe {
@@ -23,6 +25,23 @@ int check_launch(const char *what) {
     set_error("%s: %s", what, hipGetErrorString(e));
     return (int)e;
   }
+  return 0;
+}
+
+int ensure_dynamic_lds(const void *kernel, int bytes, DeviceFlags &done, const char *what) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    set_error("%s: hipGetDevice: %s (device %d)", what, hipGetErrorString(e), dev);
+    return e != hipSuccess ? (int)e : YAMOE_E_ARG;
+  }
+  if (done.flag[dev].load(std::memory_order_acquire)) return 0;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) {
+    set_error("%s: hipFuncSetAttribute(MaxDynamicSharedMemorySize=%d): %s", what, bytes, hipGetErrorString(e));
+    return (int)e;
+  }
+  done.flag[dev].store(true, std::memory_order_release);
   return 0;
 }
 

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/yamoe_hip.h"
 
 namespace yamoe {
@@ -152,5 +154,14 @@ int route_and_schedule(const void *router_indices, int32_t idx_i64, int32_t N, i
 // error reporting for the C ABI
 void set_error(const char *fmt, ...);
 int check_launch(const char *what);
+
+// Kernels that use more than 64 KB of dynamic LDS need hipFuncAttributeMaxDynamicSharedMemorySize raised, once per
+// device (every device loads its own copy of the code).  `done` holds one flag per device for one kernel; the
+// attribute call is idempotent, so two threads racing through the first call are harmless.
+constexpr int kMaxDevices = 64;
+struct DeviceFlags {
+  std::atomic<bool> flag[kMaxDevices];
+};
+int ensure_dynamic_lds(const void *kernel, int bytes, DeviceFlags &done, const char *what);
 
 }  // namespace yamoe

@@ -530,15 +530,8 @@ __global__ __launch_bounds__(kGemmThreads) void grouped_gemm_kernel(const GemmAr
 template <typename T, int A_KIND, int B_KIND, int EPI, int PROB, bool GATHER>
 static int launch_gemm(const GemmArgs &args, int max_row_tiles, hipStream_t stream) {
   auto kernel = grouped_gemm_kernel<T, A_KIND, B_KIND, EPI, PROB, GATHER>;
-  static bool attr_done = false;  // benign race: the attribute call is idempotent
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds);
-    if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(MaxDynamicSharedMemorySize=%d): %s", kGemmLds, hipGetErrorString(e));
-      return (int)e;
-    }
-    attr_done = true;
-  }
+  static DeviceFlags attr_done;  // one per kernel instantiation
+  if (int rc = ensure_dynamic_lds((const void *)kernel, kGemmLds, attr_done, "grouped_gemm_kernel")) return rc;
   long long total = (long long)max_row_tiles * args.n_col_tiles;
   if (total <= 0) return 0;
   total = (total + kXcds - 1) / kXcds * kXcds;

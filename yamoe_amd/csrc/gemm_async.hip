@@ -643,15 +643,8 @@ template <typename T, int EPI, bool GATHER, bool BNK>
 static int launch(const Args &args, int max_row_tiles, hipStream_t stream) {
   auto kernel = gemm_async_kernel<T, EPI, GATHER, BNK>;
   constexpr int lds_bytes = BNK ? (kLdsNk > kLds ? kLdsNk : kLds) : kLds;
-  static bool attr_done = false;  // benign race: the attribute call is idempotent
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(MaxDynamicSharedMemorySize=%d): %s", lds_bytes, hipGetErrorString(e));
-      return (int)e;
-    }
-    attr_done = true;
-  }
+  static DeviceFlags attr_done;  // one per kernel instantiation
+  if (int rc = ensure_dynamic_lds((const void *)kernel, lds_bytes, attr_done, "gemm_async_kernel")) return rc;
   long long total = (long long)max_row_tiles * args.n_col_tiles;
   if (total <= 0) return 0;
   total = (total + kXcds - 1) / kXcds * kXcds;
@@ -988,15 +981,8 @@ int gemm_async_wgrad(const void *L, const void *R, void *dW, const int *counts, 
   a.n_m_tiles = ceil_div(Md, async::kSmallBM);
   a.n_n_tiles = ceil_div(Nd, async::kBN);
   auto kernel = async::wgrad_small_kernel<T>;
-  static bool attr_done = false;  // benign race: the attribute call is idempotent
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, async::kSmallLds);
-    if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(MaxDynamicSharedMemorySize=%d): %s", async::kSmallLds, hipGetErrorString(e));
-      return (int)e;
-    }
-    attr_done = true;
-  }
+  static DeviceFlags attr_done;
+  if (int rc = ensure_dynamic_lds((const void *)kernel, async::kSmallLds, attr_done, "wgrad_small_kernel")) return rc;
   long long total = (long long)E * a.n_m_tiles * a.n_n_tiles;
   if (total <= 0) return 0;
   total = (total + kXcds - 1) / kXcds * kXcds;

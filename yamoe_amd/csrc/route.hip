@@ -435,17 +435,11 @@ int yamoe::route_and_schedule(const void *router_indices, int32_t idx_i64, int32
   const int buckets = E + 1;
   if (N <= kSingleBlockMaxN) {
     size_t lds = route_single_lds_bytes(N, buckets);
-    static bool attr_done = false;  // benign race: the attribute calls are idempotent
-    if (!attr_done) {
-      const int max_lds = (int)route_single_lds_bytes(kSingleBlockMaxN, kRouteMaxBuckets);
-      hipError_t e1 = hipFuncSetAttribute((const void *)route_single_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
-      hipError_t e2 = hipFuncSetAttribute((const void *)route_single_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, max_lds);
-      if (e1 != hipSuccess || e2 != hipSuccess) {
-        set_error("hipFuncSetAttribute(MaxDynamicSharedMemorySize=%d): %s", max_lds, hipGetErrorString(e1 != hipSuccess ? e1 : e2));
-        return (int)(e1 != hipSuccess ? e1 : e2);
-      }
-      attr_done = true;
-    }
+    static DeviceFlags attr_i64, attr_i32;
+    const int max_lds = (int)route_single_lds_bytes(kSingleBlockMaxN, kRouteMaxBuckets);
+    int rc = idx_i64 ? ensure_dynamic_lds((const void *)route_single_kernel<true>, max_lds, attr_i64, "route_single_kernel")
+                     : ensure_dynamic_lds((const void *)route_single_kernel<false>, max_lds, attr_i32, "route_single_kernel");
+    if (rc != 0) return rc;
     if (idx_i64)
       hipLaunchKernelGGL(route_single_kernel<true>, dim3(1), dim3(kRouteThreads), lds, stream,
                          router_indices, N, E, capacity, sorted_expert, sorted_idx, counts, offsets, inv_pos, (int *)schedule,
