@@ -119,6 +119,24 @@ int yamoe_experts_forward(const yamoe_problem *p, const void *hidden_states,
                           const void *down_proj, const void *down_proj_bias, void *out,
                           void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- the whole forward without a workspace argument -------------------------------------------
+ * No counterpart in the reference.  For callers that cannot allocate device memory at all, not even
+ * a workspace: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * Same arguments, kernels and results as yamoe_experts_forward, but the workspace is an array of
+ * YAMOE_STATIC_SCRATCH_BYTES that is part of the library's device image (each GPU the library runs
+ * on holds its copy until the process ends).  The call allocates and frees nothing; its first call
+ * on a device looks the array's address up (one hipGetSymbolAddress).  Problems whose
+ * yamoe_experts_workspace_bytes() exceeds the array are rejected with YAMOE_E_WORKSPACE (at
+ * H = I = 2880 in a 16-bit dtype the limit is about 2900 (token, expert) assignments, e.g. 725
+ * tokens at top-4).  All calls on one GPU share that GPU's array: two calls whose work overlaps on
+ * the same GPU (different streams, or different threads) race; calls on one stream are ordered. */
+#define YAMOE_STATIC_SCRATCH_BYTES (32u << 20)
+int yamoe_experts_forward_static(const yamoe_problem *p, const void *hidden_states,
+                                 const void *router_indices, const void *routing_weights,
+                                 const void *gate_up_proj, const void *gate_up_proj_bias,
+                                 const void *down_proj, const void *down_proj_bias, void *out,
+                                 void *stream);
+
 /* ---- the whole backward: experts_backward_cuda (csrc/experts_backward.cu:126-341)
  * Outputs (all fully written, caller need not zero them):
  *   d_hidden [T,H], d_routing [T,rw_cols] (zero outside the selected experts),

@@ -1,0 +1,59 @@
+"""yamoe_experts_forward_static: the forward on the workspace that is built into the library, through the C ABI.
+
+It runs the kernels of yamoe_experts_forward on a different workspace address, so its output must equal that entry
+point's bit for bit; checked on two calls in a row, the second on a smaller problem (the array then still holds the
+first call's lists and rows), and once more after the first problem again.  Problems beyond the array are refused."""
+import ctypes
+
+import pytest
+import torch
+
+from tests.util import KEYS
+from yamoe_amd.workloads import make_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def both(d, capacity, gpu):
+    from yamoe_amd import _cabi
+    g = [d[k].to(gpu) for k in KEYS]
+    want = _cabi.experts_forward(*g, capacity)
+    got = torch.full_like(want, float("nan"))
+    before = torch.cuda.memory_allocated()
+    _cabi.experts_forward_static(*g, capacity, got)
+    assert torch.cuda.memory_allocated() == before
+    torch.cuda.synchronize()
+    return got.cpu(), want.cpu()
+
+
+def test_static_workspace_forward_matches(gpu):
+    from oracle import yamoe_oracle as O
+    big = make_inputs(700, 256, 192, 8, 2, torch.bfloat16, seed=51, w_std=0.05, bias_std=0.1, zipf=0.8)   # tiles and streamed experts
+    small = make_inputs(40, 128, 64, 4, 2, torch.bfloat16, seed=52, w_std=0.05, bias_std=0.1)
+    for label, d, cap in (("first", big, 700), ("second, smaller", small, 40), ("first again, capacity 100", big, 100)):
+        print("static workspace:", label, flush=True)
+        got, want = both(d, cap, gpu)
+        assert torch.equal(got, want), label
+        ref = O.experts_capacity(*[d[k] for k in KEYS], cap, compute_dtype=torch.float32)
+        assert O.rel_l2(got, ref) < 1e-2
+
+
+def test_static_workspace_forward_fp32_and_decode_shape(gpu):
+    d = make_inputs(300, 64, 96, 4, 2, torch.float32, seed=53, w_std=0.05, bias_std=0.1)
+    got, want = both(d, 300, gpu)
+    assert torch.equal(got, want)
+    d = make_inputs(64, 2880, 2880, 8, 4, torch.bfloat16, seed=54)    # the decode expert shape, 256 assignments
+    got, want = both(d, 64, gpu)
+    assert torch.equal(got, want)
+
+
+def test_static_workspace_forward_refuses_large_problems(gpu):
+    from yamoe_amd import _cabi
+    T, H, I, E, K = 4096, 2880, 2880, 2, 4
+    p = _cabi.Problem(T=T, K=K, E=E, H=H, I=I, capacity=T, dtype=_cabi.BF16, idx_i64=1, rw_cols=E)
+    assert _cabi.lib().yamoe_experts_workspace_bytes(ctypes.byref(p)) > _cabi.STATIC_SCRATCH_BYTES
+    one = torch.zeros(1, device=gpu)
+    ptr = ctypes.c_void_p(one.data_ptr())   # never touched: the size check comes first
+    rc = _cabi.lib().yamoe_experts_forward_static(ctypes.byref(p), *([ptr] * 8), ptr, None)
+    assert rc == -2, rc   # YAMOE_E_WORKSPACE
+    assert b"built-in" in _cabi.lib().yamoe_last_error()

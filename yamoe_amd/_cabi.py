@@ -19,7 +19,8 @@ _DTYPE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 SYMBOLS = [
     "yamoe_abi_version", "yamoe_last_error", "yamoe_route_workspace_bytes", "yamoe_route", "yamoe_permute",
     "yamoe_combine", "yamoe_schedule_bytes", "yamoe_build_schedule", "yamoe_gate_up", "yamoe_down",
-    "yamoe_experts_workspace_bytes", "yamoe_experts_forward", "yamoe_experts_backward_workspace_bytes",
+    "yamoe_experts_workspace_bytes", "yamoe_experts_forward", "yamoe_experts_forward_static",
+    "yamoe_experts_backward_workspace_bytes",
     "yamoe_experts_backward", "yamoe_sort_workspace_bytes", "yamoe_sort", "yamoe_bincount_cumsum", "yamoe_padded_gather",
     "yamoe_padded_scatter_workspace_bytes", "yamoe_padded_scatter", "yamoe_index_select", "yamoe_regular_groups",
     "yamoe_batch_mm_workspace_bytes", "yamoe_batch_mm", "yamoe_router_topk",
@@ -56,6 +57,7 @@ def lib():
         L.yamoe_experts_workspace_bytes.restype = sz
         L.yamoe_experts_workspace_bytes.argtypes = [pp]
         L.yamoe_experts_forward.argtypes = [pp] + [vp] * 9 + [sz, vp]
+        L.yamoe_experts_forward_static.argtypes = [pp] + [vp] * 8 + [vp]
         L.yamoe_experts_backward_workspace_bytes.restype = sz
         L.yamoe_experts_backward_workspace_bytes.argtypes = [pp]
         L.yamoe_experts_backward.argtypes = [pp] + [vp] * 15 + [sz, vp]
@@ -197,4 +199,19 @@ def experts_forward(hidden, router_indices, routing_weights, gate_up_proj, gate_
     _check(lib().yamoe_experts_forward(ctypes.byref(p), _p(hidden), _p(router_indices), _p(routing_weights),
                                        _p(gate_up_proj), _p(gate_up_proj_bias), _p(down_proj), _p(down_proj_bias),
                                        _p(out), _p(workspace), workspace.numel(), _stream()), "yamoe_experts_forward")
+    return out
+
+
+STATIC_SCRATCH_BYTES = 32 << 20  # YAMOE_STATIC_SCRATCH_BYTES of include/yamoe_hip.h
+
+
+def experts_forward_static(hidden, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
+                           down_proj_bias, capacity, out):
+    """yamoe_experts_forward_static: the forward on the library's built-in workspace; allocates nothing (`out` is the
+    caller's)."""
+    _need_gpu(hidden, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj, down_proj_bias, out)
+    p = problem(hidden, router_indices, routing_weights, gate_up_proj, capacity)
+    _check(lib().yamoe_experts_forward_static(ctypes.byref(p), _p(hidden), _p(router_indices), _p(routing_weights),
+                                              _p(gate_up_proj), _p(gate_up_proj_bias), _p(down_proj),
+                                              _p(down_proj_bias), _p(out), _stream()), "yamoe_experts_forward_static")
     return out

@@ -428,6 +428,60 @@ extern "C" int yamoe_experts_forward(const yamoe_problem *p, const void *hidden_
                                            (hipStream_t)stream));
 }
 
+// ---- the forward without a workspace argument ----------------------------------------------------------
+// The workspace of yamoe_experts_forward_static: one array per GPU, part of the loaded code object, so no call ever
+// allocates it.  In host code the array's name is only a handle for hipGetSymbolAddress; the address the kernels get
+// is looked up once per device (with that device current) and kept.  Every call on a GPU uses that GPU's array.
+static __device__ __align__(256) unsigned char scratch[YAMOE_STATIC_SCRATCH_BYTES];
+static std::atomic<void *> g_scratch_ptr[kMaxDevices];
+
+static int static_scratch(void **out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    set_error("yamoe_experts_forward_static: hipGetDevice: %s (device %d)", hipGetErrorString(e), dev);
+    return e != hipSuccess ? (int)e : YAMOE_E_ARG;
+  }
+  void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      set_error("yamoe_experts_forward_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+      return e != hipSuccess ? (int)e : YAMOE_E_ARG;
+    }
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // two first callers find the same address
+  }
+  *out = ptr;
+  return 0;
+}
+
+extern "C" int yamoe_experts_forward_static(const yamoe_problem *p, const void *hidden_states,
+                                            const void *router_indices, const void *routing_weights,
+                                            const void *gate_up_proj, const void *gate_up_proj_bias,
+                                            const void *down_proj, const void *down_proj_bias, void *out,
+                                            void *stream) {
+  YAMOE_TRY(check_problem(p, "yamoe_experts_forward_static"));
+  if (p->T == 0) return 0;
+  if (!hidden_states || !router_indices || !routing_weights || !gate_up_proj || !gate_up_proj_bias || !down_proj ||
+      !down_proj_bias || !out) {
+    set_error("yamoe_experts_forward_static: null pointer");
+    return YAMOE_E_ARG;
+  }
+  const size_t need = yamoe_experts_workspace_bytes(p);
+  if (need > (size_t)YAMOE_STATIC_SCRATCH_BYTES) {
+    set_error("yamoe_experts_forward_static: this problem needs %zu bytes of workspace, the built-in one holds %zu "
+              "(T*K*(I + max(H,I)) elements plus the routing lists); use yamoe_experts_forward with a caller-owned "
+              "workspace", need, (size_t)YAMOE_STATIC_SCRATCH_BYTES);
+    return YAMOE_E_WORKSPACE;
+  }
+  void *ws = nullptr;
+  YAMOE_TRY(static_scratch(&ws));
+  // Nothing in the workspace has to start at zero: every list, counter and row the kernels read is written earlier
+  // in the same call, so the contents left by the previous call on this GPU do not matter.
+  YAMOE_DISPATCH(p->dtype, forward_impl<T>(p, hidden_states, router_indices, routing_weights, gate_up_proj,
+                                           gate_up_proj_bias, down_proj, down_proj_bias, out, ws, (hipStream_t)stream));
+}
+
 extern "C" size_t yamoe_experts_backward_workspace_bytes(const yamoe_problem *p) {
   if (check_problem(p, "yamoe_experts_backward_workspace_bytes")) return 0;
   BackwardBuffers b;
