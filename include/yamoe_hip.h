@@ -61,7 +61,8 @@ const char *yamoe_last_error(void);
  *   offsets        [E+1] exclusive prefix sum of counts; offsets[E] = number of valid ids
  *   inv_pos        [N]  sorted position of each flat slot, or -1 when the slot is
  *                       dropped (rank inside its expert >= capacity, or id outside [0,E))
- * Ids outside [0,E) sort after every valid expert. */
+ * Ids outside [0,E) sort after every valid expert.  Limit: E <= 768 (this bounds every entry point
+ * that routes: the whole forward and backward too). */
 size_t yamoe_route_workspace_bytes(int32_t N, int32_t E);
 int yamoe_route(const void *router_indices, int32_t idx_i64, int32_t N, int32_t E,
                 int32_t capacity, int32_t *sorted_expert, int32_t *sorted_idx,
@@ -111,7 +112,9 @@ int yamoe_down(const void *act, const void *down_proj, const void *down_proj_bia
                const void *schedule, int32_t N, int32_t E, int32_t H, int32_t I, int32_t dtype,
                void *stream);
 
-/* ---- the whole forward: experts_cuda (csrc/moe.cpp:45-223) ------------------- */
+/* ---- the whole forward: experts_cuda (csrc/moe.cpp:45-223) -------------------
+ * Limits (YAMOE_E_ARG otherwise): H and I multiples of 8 (16-bit dtypes) or 4 (fp32); E <= 768;
+ * T*K < 2^30; hidden_states (and grad_out) below 4 GiB. */
 size_t yamoe_experts_workspace_bytes(const yamoe_problem *p);
 int yamoe_experts_forward(const yamoe_problem *p, const void *hidden_states,
                           const void *router_indices, const void *routing_weights,
@@ -163,7 +166,8 @@ int yamoe_sort(const void *x, int32_t elem_bytes, int32_t n, int32_t end_bit, vo
                void *iota_out, void *workspace, size_t workspace_bytes, void *stream);
 
 /* bincount_cumsum_cuda (csrc/bincount_cumsum.cu:58-97): output[b] = number of inputs <= b for
- * b < minlength (inclusive prefix sum of the bin counts); output[minlength..output_len) = 0. */
+ * b < minlength (inclusive prefix sum of the bin counts); output[minlength..output_len) = 0.
+ * Limit: minlength <= 8192 bins. */
 int yamoe_bincount_cumsum(const int32_t *input, int32_t n, int32_t *output, int32_t output_len,
                           int32_t minlength, void *stream);
 

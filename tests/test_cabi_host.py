@@ -43,6 +43,16 @@ def test_size_queries_and_validation_need_no_gpu():
         q = _cabi.Problem(**{**{f: getattr(p, f) for f, _ in p._fields_}, **bad})
         assert lib.yamoe_experts_workspace_bytes(ctypes.byref(q)) == 0
         assert len(lib.yamoe_last_error()) > 0
+    # hidden_states of 4 GiB or more: token rows are gathered with 32-bit byte offsets from the tensor's start
+    for T_big, dt, ok in ((745000, _cabi.BF16, True), (746000, _cabi.BF16, False), (372000, _cabi.F32, True),
+                          (373000, _cabi.F32, False)):
+        q = _cabi.Problem(**{**{f: getattr(p, f) for f, _ in p._fields_}, **dict(T=T_big, capacity=T_big, dtype=dt)})
+        assert (lib.yamoe_experts_workspace_bytes(ctypes.byref(q)) > 0) == ok, (T_big, dt)
+        if not ok:
+            assert b"4 GiB" in lib.yamoe_last_error()
+            assert lib.yamoe_experts_backward_workspace_bytes(ctypes.byref(q)) == 0
+    rc = lib.yamoe_gate_up(None, None, None, None, None, None, None, 746000 * 4, 4, 32, 2880, 2880, _cabi.BF16, None)
+    assert rc == -1
     # yamoe_route rejects too many experts before any launch
     rc = lib.yamoe_route(None, 1, 0, 100000, 1, None, None, None, None, None, None, 0, None)
     assert rc == -1 and b"yamoe_route" in lib.yamoe_last_error()
