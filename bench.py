@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Benchmark of the expert-layer forward on one MI355X.
+"""Benchmark of the expert-layer path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
@@ -11,11 +11,15 @@ already resident in HBM.  Prints ONE JSON line.  `value` is algorithmic TFLOP/s 
 Also on the line:
   roofline      the dominant kernel (the gate_up grouped GEMM), timed on its own with HIP events on
                 the stream it runs on: algorithmic flop per launch / average launch time vs the
-                2.5 PFLOP/s dense bf16 MFMA peak
-  decode        the 64-token / 128-expert decode workload: algorithmic HBM bytes per step / step time
-                vs the 8 TB/s HBM peak
+                2.5 PFLOP/s dense bf16 MFMA peak; `traffic` (HBM bytes per launch) is read from the
+                counter summary kept under profiles/ and says so
   cpu_baseline  the CPU oracle (oracle/yamoe_oracle.py, the loop-over-experts path the reference itself
-                takes on a CPU) timed on this box's host cores on a slice of the same batch
+                takes on a CPU) timed on this box's host cores on the same batch
+  parity        the timed op's output against that oracle run
+  configs       all five measured workloads, each with its time, its rate against its own peak (fp32 or bf16
+                MFMA, HBM for the decode shape) and its parity against the oracle:
+                cfg1 README shape fp32, cfg2 the headline, cfg3 decode, cfg4 Zipf-skewed, cfg5 backward
+  decode        the cfg3 entry again under the name the metric gives it
 """
 import argparse
 import json
@@ -30,12 +34,11 @@ sys.path.insert(0, ROOT)
 # object on the same line carries the second (GB/s and fraction of HBM peak)
 METRIC = "experts() fwd TFLOP/s & %MFMA peak (20B shape, 4096 tok); decode GB/s %HBM"
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_FP32_TFLOPS = 157.3   # MI355X fp32 matrix
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
-
-# HBM bytes per launch of the gate_up GEMM on the GPT-OSS-20B workload, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs of this file (profiles/gemm_async_and_stream_gemm_counters.md): 713 500 KiB fetched x 2.0
-# (FETCH_SIZE reads half of a 1 GiB copy's bytes on this device) + 94 046 KiB written x 1.0.
-GATE_UP_TRAFFIC_BYTES = 1.627e9
+ORDER = ("hidden", "router_indices", "routing_weights", "gate_up_proj", "gate_up_proj_bias", "down_proj",
+         "down_proj_bias")
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gate_up_traffic.json")
 
 
 def spin_up(fn, ms):
@@ -66,18 +69,20 @@ def event_time_ms(fn, iters):
     return start.elapsed_time(end) / iters
 
 
-def device_weights(E, H, I, dtype, std, seed, device):
-    """Weights drawn on the device (N(0, std)); used where drawing on the host would take minutes."""
-    import torch
-    g = torch.Generator(device=device).manual_seed(seed)
+def parity_of(got, want, tol, against):
+    from oracle import yamoe_oracle as O
+    return dict(rel_l2=float("%.3e" % O.rel_l2(got, want)), max_abs=float("%.3e" % O.max_abs(got, want)),
+                tolerance=tol, against=against)
 
-    def draw(shape):
-        t = torch.empty(shape, dtype=dtype, device=device)
-        for e in range(shape[0]):
-            t[e] = (torch.randn(shape[1:], generator=g, device=device) * std).to(dtype)
-        return t
-    return dict(gate_up_proj=draw((E, H, 2 * I)), gate_up_proj_bias=draw((E, 2 * I)), down_proj=draw((E, I, H)),
-                down_proj_bias=draw((E, H)))
+
+def recorded_traffic():
+    """HBM bytes per launch of the gate_up GEMM from the committed counter summary (not measured by this run)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            t = json.load(f)
+        return float(t["bytes_per_launch"]), "profiles/gate_up_traffic.json (%s)" % t.get("from", "counter run")
+    except (OSError, KeyError, ValueError):
+        return None, None
 
 
 def main():
@@ -87,10 +92,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--spinup-ms", type=float, default=1000.0,
                     help="untimed load before each timed region so that the engine clock has left its idle state")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle (no cpu_baseline, no parity)")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="only the headline workload and its dominant kernel (for profiler runs)")
+    ap.add_argument("--only", default="", help="with --no-configs: also run this one of decode, zipf, readme, backward")
     ap.add_argument("--extras", action="store_true",
-                    help="also time the backward (GPT-OSS-20B shape), the Zipf-skewed and the README fp32 workloads")
+                    help="also time the vendor library's dense GEMM on the two forward GEMM shapes, and the routing "
+                         "and permute kernels of the Zipf workload on their own")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy kernel (a known FETCH_SIZE / WRITE_SIZE for counter runs)")
     args = ap.parse_args()
@@ -104,12 +112,20 @@ def main():
 
     import yamoe_amd
     from yamoe_amd import _cabi, workloads
+    from yamoe_amd.workloads import device_weights
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    torch.set_num_threads(min(os.cpu_count() or 1, 16))
+    check = not args.no_cpu_baseline
+    if check:
+        from oracle import yamoe_oracle as O
+
+    def wanted(name):
+        return not args.no_configs or args.only == name
 
     if args.calibrate_copy:
         src = torch.ones(1 << 28, dtype=torch.float32, device=dev)  # 1 GiB
@@ -118,15 +134,15 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    # ---------------- GPT-OSS-20B shaped layer ----------------------------------------------------------
+    configs = {}
+
+    # ---------------- cfg2: GPT-OSS-20B shaped layer (the headline) --------------------------------------
     cfg = workloads.CONFIGS["gptoss20b"]
     T, H, I, E, K = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["K"]
     host, _ = workloads.make_config("gptoss20b", seed=0, weights=False)
     d = {k: v.to(dev) for k, v in host.items()}
     d.update(device_weights(E, H, I, torch.bfloat16, cfg["w_std"], 1, dev))
-    order = ("hidden", "router_indices", "routing_weights", "gate_up_proj", "gate_up_proj_bias", "down_proj",
-             "down_proj_bias")
-    a = [d[k] for k in order]
+    a = [d[k] for k in ORDER]
     n_rows = T * K  # capacity = T keeps every assignment
     flop = n_rows * workloads.FWD_FLOP_PER_ROW(H, I)
 
@@ -165,24 +181,24 @@ def main():
     gu_flop = n_rows * 4 * H * I
     gu_tflops = gu_flop / (gu_ms * 1e-3) / 1e12
     dn_tflops = n_rows * 2 * H * I / (dn_ms * 1e-3) / 1e12
+    traffic, traffic_source = recorded_traffic()
     roofline = dict(bound="mfma", kernel="gemm_async_kernel<bf16, gate_up + clamped SwiGLU>", achieved=round(gu_tflops, 2),
                     peak=PEAK_BF16_TFLOPS, unit="TFLOP/s", frac=round(gu_tflops / PEAK_BF16_TFLOPS, 4),
-                    traffic=GATE_UP_TRAFFIC_BYTES, avg_launch_ms=round(gu_ms, 4),
+                    traffic=traffic, traffic_source=traffic_source, algorithmic_flop_per_launch=gu_flop,
+                    avg_launch_ms=round(gu_ms, 4),
                     down_gemm=dict(achieved=round(dn_tflops, 2), frac=round(dn_tflops / PEAK_BF16_TFLOPS, 4),
                                    avg_launch_ms=round(dn_ms, 4)))
+    del act, y
 
-    # ---------------- CPU baseline on a slice of the same batch ------------------------------------------
+    # ---------------- CPU baseline on the same batch, and the parity of the timed op ---------------------
     cpu_baseline = None
     parity = None
-    if not args.no_cpu_baseline:
-        from oracle import yamoe_oracle as O
-        sample_tokens = T  # the whole batch; repeated until about 10 s of CPU work have been timed
-        torch.set_num_threads(min(os.cpu_count() or 1, 16))
+    hs = None
+    if check:
         # inputs are converted to the fp32 compute type once, outside the timed region
-        hs = {k: d[k][:sample_tokens].cpu() if k in ("hidden", "router_indices", "routing_weights") else d[k].cpu()
-              for k in order}
+        hs = {k: d[k].cpu() for k in ORDER}
         hs = {k: (v.float() if v.is_floating_point() else v) for k, v in hs.items()}
-        hargs = [hs[k] for k in order]
+        hargs = [hs[k] for k in ORDER]
         O.experts_loop(*[t[:64] if i < 3 else t for i, t in enumerate(hargs)], compute_dtype=torch.float32)  # warm-up
         times = []
         while len(times) < 3 or sum(times) < 10.0:
@@ -190,26 +206,51 @@ def main():
             ref = O.experts_loop(*hargs, compute_dtype=torch.float32)
             times.append(time.perf_counter() - t1)
         cpu_s = sorted(times)[len(times) // 2]
-        cpu_flop = sample_tokens * K * workloads.FWD_FLOP_PER_ROW(H, I)
-        cpu_baseline = dict(value=round(cpu_flop / cpu_s / 1e12, 4), unit="TFLOP/s", cores=torch.get_num_threads(),
+        cpu_baseline = dict(value=round(flop / cpu_s / 1e12, 4), unit="TFLOP/s", cores=torch.get_num_threads(),
                             kind="port", sample="all %d tokens of the same batch, fp32 compute on the bf16 inputs, "
-                            "median of %d runs (%.2f s each, %.1f s in all)" % (sample_tokens, len(times), cpu_s, sum(times)))
-        got = step()[:sample_tokens].float().cpu()
-        parity = dict(rel_l2=float("%.3e" % O.rel_l2(got, ref)), max_abs=float("%.3e" % O.max_abs(got, ref)),
-                      tolerance=1e-2, against="fp32 oracle on all %d tokens" % sample_tokens)
-        del hs, hargs
+                            "median of %d runs (%.2f s each, %.1f s in all)" % (T, len(times), cpu_s, sum(times)))
+        parity = parity_of(step().float().cpu(), ref, 1e-2, "fp32 oracle on all %d tokens" % T)
+        del ref
+    configs["cfg2_gptoss20b_forward_bf16"] = dict(
+        ms=round(ms_per_step, 4), tflops=round(value, 2), frac_of_peak=round(value / PEAK_BF16_TFLOPS, 4),
+        peak="bf16 MFMA %.0f TFLOP/s" % PEAK_BF16_TFLOPS, parity=parity)
 
-    # ---------------- decode workload: 64 tokens, 128 experts ---------------------------------------------
+    def timed(fn, iters):
+        spin_up(fn, args.spinup_ms)
+        return event_time_ms(fn, iters)
+
+    few = max(3, args.steps // 4)
+
+    # ---------------- cfg5: backward at the same shape ------------------------------------------------------
+    if wanted("backward"):
+        gy = torch.randn(T, H, device=dev, generator=torch.Generator(device=dev).manual_seed(3)).to(torch.bfloat16)
+        ms = timed(lambda: yamoe_amd.experts_backward(gy, *a, T, E, K), few)
+        b_flop = n_rows * 18 * H * I  # forward recompute 6 + input gradients 6 + weight gradients 6 (per assignment, x H*I)
+        tf = b_flop / (ms * 1e-3) / 1e12
+        entry = dict(ms=round(ms, 4), tflops=round(tf, 2), frac_of_peak=round(tf / PEAK_BF16_TFLOPS, 4),
+                     peak="bf16 MFMA %.0f TFLOP/s" % PEAK_BF16_TFLOPS, algorithmic_flop=b_flop, parity=None)
+        if check:
+            grads = [g.float().cpu() for g in yamoe_amd.experts_backward(gy, *a, T, E, K)]
+            want = O.experts_backward(gy.cpu(), *[hs[k] for k in ORDER], T, compute_dtype=torch.float32)
+            names = ("d_hidden", "d_routing", "d_gate_up_proj", "d_gate_up_proj_bias", "d_down_proj", "d_down_proj_bias")
+            per = {n: float("%.3e" % O.rel_l2(g, w)) for n, g, w in zip(names, grads, want)}
+            entry["parity"] = dict(rel_l2=max(per.values()), per_gradient=per, tolerance=1e-2,
+                                   against="fp32 autograd through the oracle, all six gradients (worst shown)")
+            del grads, want
+        configs["cfg5_gptoss20b_backward_bf16"] = entry
+        del gy
+    del d, a, hs
+    torch.cuda.empty_cache()
+
+    # ---------------- cfg3: decode, 64 tokens, 128 experts ---------------------------------------------------
     decode = None
-    if not args.no_decode:
-        del d, a, act, y
-        torch.cuda.empty_cache()
+    if wanted("decode"):
         dc = workloads.CONFIGS["decode"]
         Td, Ed, Kd = dc["T"], dc["E"], dc["K"]
         hostd, _ = workloads.make_config("decode", seed=0, weights=False)
         dd = {k: v.to(dev) for k, v in hostd.items()}
         dd.update(device_weights(Ed, H, I, torch.bfloat16, dc["w_std"], 2, dev))
-        ad = [dd[k] for k in order]
+        ad = [dd[k] for k in ORDER]
         n_active = int((np.bincount(hostd["router_indices"].numpy().ravel(), minlength=Ed) > 0).sum())
         nbytes = workloads.algorithmic_bytes_decode(n_active, Td, Kd, Ed, H, I)
 
@@ -223,77 +264,82 @@ def main():
         gbs = nbytes / (d_ms * 1e-3) / 1e9
         decode = dict(metric="experts_fwd_decode_hbm_gbs", value=round(gbs, 1), unit="GB/s", ms_per_step=round(d_ms, 4),
                       frac_of_hbm_peak=round(gbs / PEAK_HBM_GBS, 4), peak=PEAK_HBM_GBS, active_experts=n_active,
-                      algorithmic_bytes=nbytes,
+                      algorithmic_bytes=nbytes, parity=None,
                       config=dict(workload="decode: T=64 H=I=2880 E=128 top-4 bf16", tokens=Td, experts=Ed, top_k=Kd))
-
-    extras = None
-    if args.extras:
-        extras = {}
-        try:
-            del dd, ad
-        except NameError:
-            del d, a, act, y
+        if check:
+            want = O.experts_capacity(*[dd[k].cpu() for k in ORDER], Td, compute_dtype=torch.float32)
+            decode["parity"] = parity_of(dstep().float().cpu(), want, 1e-2, "fp32 oracle, all 64 tokens, device-drawn weights copied back")
+        configs["cfg3_decode_bf16"] = dict(ms=round(d_ms, 4), gbs=round(gbs, 1), frac_of_peak=round(gbs / PEAK_HBM_GBS, 4),
+                                           peak="HBM %.0f GB/s" % PEAK_HBM_GBS, parity=decode["parity"])
+        del dd, ad
         torch.cuda.empty_cache()
 
-        def timed(fn, n_flop, label, iters=max(3, args.steps // 4)):
-            spin_up(fn, args.spinup_ms)
-            ms = event_time_ms(fn, iters)
-            extras[label] = dict(ms=round(ms, 4), tflops=round(n_flop / (ms * 1e-3) / 1e12, 2),
-                                 frac_of_peak=round(n_flop / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4))
-
-        # backward at the GPT-OSS-20B shape: 18*H*I flop per assignment (forward recompute + dgrad + wgrad)
-        hostb, _ = workloads.make_config("gptoss20b", seed=0, weights=False)
-        db = {k: v.to(dev) for k, v in hostb.items()}
-        db.update(device_weights(E, H, I, torch.bfloat16, cfg["w_std"], 1, dev))
-        ab = [db[k] for k in order]
-        gy = torch.randn(T, H, device=dev, generator=torch.Generator(device=dev).manual_seed(3)).to(torch.bfloat16)
-        timed(lambda: yamoe_amd.experts_backward(gy, *ab, T, E, K), T * K * 18 * H * I, "backward_gptoss20b_bf16")
-        del db, ab, gy
-        torch.cuda.empty_cache()
-        # Zipf-skewed routing, 16384 tokens, 128 experts
+    # ---------------- cfg4: Zipf-skewed routing, 16384 tokens, 128 experts -----------------------------------
+    extras = {} if args.extras else None
+    if wanted("zipf"):
         zc = workloads.CONFIGS["zipf"]
         hostz, _ = workloads.make_config("zipf", seed=0, weights=False)
         dz = {k: v.to(dev) for k, v in hostz.items()}
         dz.update(device_weights(zc["E"], H, I, torch.bfloat16, zc["w_std"], 4, dev))
-        az = [dz[k] for k in order]
-        timed(lambda: yamoe_amd.experts(*az, zc["T"], zc["E"], zc["K"]), zc["T"] * zc["K"] * 6 * H * I,
-              "forward_zipf_bf16")
-        cz = np.bincount(hostz["router_indices"].numpy().ravel(), minlength=zc["E"])
+        az = [dz[k] for k in ORDER]
         n_z = zc["T"] * zc["K"]
+        ms = timed(lambda: yamoe_amd.experts(*az, zc["T"], zc["E"], zc["K"]), few)
+        cz = np.bincount(hostz["router_indices"].numpy().ravel(), minlength=zc["E"])
         w_bytes = int((cz > 0).sum()) * 3 * H * I * 2               # weights of the non-empty experts, read once
-        roof_ms = max(n_z * 6 * H * I / (PEAK_BF16_TFLOPS * 1e12), w_bytes / (PEAK_HBM_GBS * 1e9)) * 1e3
-        extras["forward_zipf_bf16"].update(max_rows=int(cz.max()), empty_experts=int((cz == 0).sum()),
-                                           roofline_ms=round(roof_ms, 4))
-        # its routing kernels (three launches at this N) and the row permute on their own
-        r_ms = event_time_ms(lambda: _cabi.route(dz["router_indices"], zc["E"], zc["T"]), 50)
-        se_z, si_z, _, _, _ = _cabi.route(dz["router_indices"], zc["E"], zc["T"])
-        p_ms = event_time_ms(lambda: _cabi.permute(dz["hidden"], si_z, zc["K"]), 50)
-        extras["routing_zipf"] = dict(assignments=n_z, route_ms=round(r_ms, 4), permute_ms=round(p_ms, 4),
-                                      permute_gbs=round((2 * n_z * H * 2 + 4 * n_z) / (p_ms * 1e-3) / 1e9, 1))
-        del se_z, si_z
+        z_flop = n_z * 6 * H * I
+        roof_ms = max(z_flop / (PEAK_BF16_TFLOPS * 1e12), w_bytes / (PEAK_HBM_GBS * 1e9)) * 1e3
+        tf = z_flop / (ms * 1e-3) / 1e12
+        entry = dict(ms=round(ms, 4), tflops=round(tf, 2), frac_of_peak=round(tf / PEAK_BF16_TFLOPS, 4),
+                     peak="bf16 MFMA %.0f TFLOP/s" % PEAK_BF16_TFLOPS, max_rows=int(cz.max()),
+                     empty_experts=int((cz == 0).sum()), roofline_ms=round(roof_ms, 4), parity=None)
+        if check:
+            got = yamoe_amd.experts(*az, zc["T"], zc["E"], zc["K"]).float().cpu()
+            want = O.experts_capacity(*[dz[k].cpu() for k in ORDER], zc["T"], compute_dtype=torch.float32)
+            entry["parity"] = parity_of(got, want, 1e-2, "fp32 oracle, all 16384 tokens, device-drawn weights copied back")
+            del got, want
+        configs["cfg4_zipf_forward_bf16"] = entry
+        if args.extras:
+            # its routing kernels (three launches at this N) and the row permute on their own
+            r_ms = event_time_ms(lambda: _cabi.route(dz["router_indices"], zc["E"], zc["T"]), 50)
+            se_z, si_z, _, _, _ = _cabi.route(dz["router_indices"], zc["E"], zc["T"])
+            p_ms = event_time_ms(lambda: _cabi.permute(dz["hidden"], si_z, zc["K"]), 50)
+            extras["routing_zipf"] = dict(assignments=n_z, route_ms=round(r_ms, 4), permute_ms=round(p_ms, 4),
+                                          permute_gbs=round((2 * n_z * H * 2 + 4 * n_z) / (p_ms * 1e-3) / 1e9, 1))
+            del se_z, si_z
         del dz, az
         torch.cuda.empty_cache()
-        # README shape, fp32 (peak 157.3 TFLOP/s fp32 MFMA)
+
+    # ---------------- cfg1: README shape, fp32 -----------------------------------------------------------------
+    if wanted("readme"):
         rc = workloads.CONFIGS["readme"]
         hostr, _ = workloads.make_config("readme", seed=42, weights=False)
         dr = {k: v.to(dev) for k, v in hostr.items()}
-        dr.update(device_weights(rc["E"], H, I, torch.float32, 1.0, 5, dev))
-        dr["gate_up_proj_bias"].zero_()
-        dr["down_proj_bias"].zero_()
-        ar = [dr[k] for k in order]
-        timed(lambda: yamoe_amd.experts(*ar, rc["T"], rc["E"], rc["K"]), rc["T"] * rc["K"] * 6 * H * I,
-              "forward_readme_fp32")
-        extras["forward_readme_fp32"]["frac_of_peak"] = round(extras["forward_readme_fp32"]["tflops"] / 157.3, 4)
-
+        dr.update(device_weights(rc["E"], H, I, torch.float32, 1.0, 5, dev, bias_std=0.0))
+        ar = [dr[k] for k in ORDER]
+        ms = timed(lambda: yamoe_amd.experts(*ar, rc["T"], rc["E"], rc["K"]), few)
+        r_flop = rc["T"] * rc["K"] * 6 * H * I
+        tf = r_flop / (ms * 1e-3) / 1e12
+        entry = dict(ms=round(ms, 4), tflops=round(tf, 2), frac_of_peak=round(tf / PEAK_FP32_TFLOPS, 4),
+                     peak="fp32 MFMA %.1f TFLOP/s" % PEAK_FP32_TFLOPS, parity=None)
+        if check:
+            got = yamoe_amd.experts(*ar, rc["T"], rc["E"], rc["K"]).cpu()
+            want = O.experts_capacity(*[dr[k].cpu() for k in ORDER], rc["T"], compute_dtype=torch.float64)
+            entry["parity"] = parity_of(got, want, 1e-5, "fp64 oracle, all 4096 tokens, device-drawn weights copied back")
+            del got, want
+        configs["cfg1_readme_forward_fp32"] = entry
         del dr, ar
         torch.cuda.empty_cache()
+
+    if args.extras:
         # For scale: the vendor library's dense GEMM (torch.matmul) on the same flop counts and operand layouts as the
         # two forward GEMMs: [T*K, H] x [H, 2I] and [T*K, I] x [I, H], one matrix instead of 32 experts, no bias, no GLU.
         gl = torch.Generator(device=dev).manual_seed(7)
         xa = torch.randn(T * K, H, device=dev, generator=gl).to(torch.bfloat16)
         for label, n_out in (("library_dense_gemm_gate_up_shape", 2 * I), ("library_dense_gemm_down_shape", H)):
             wb = (torch.randn(H, n_out, device=dev, generator=gl) * 0.02).to(torch.bfloat16)
-            timed(lambda: torch.matmul(xa, wb), 2 * T * K * H * n_out, label)
+            ms = timed(lambda: torch.matmul(xa, wb), few)
+            tf = 2 * T * K * H * n_out / (ms * 1e-3) / 1e12
+            extras[label] = dict(ms=round(ms, 4), tflops=round(tf, 2), frac_of_peak=round(tf / PEAK_BF16_TFLOPS, 4))
             del wb
         del xa
 
@@ -304,7 +350,7 @@ def main():
                             tokens=T, hidden=H, intermediate=I, experts=E, top_k=K,
                             algorithmic_flop=flop),
                 frac_of_mfma_peak=round(value / PEAK_BF16_TFLOPS, 4), roofline=roofline, cpu_baseline=cpu_baseline,
-                parity=parity, decode=decode, extras=extras)
+                parity=parity, decode=decode, configs=configs, extras=extras)
     print(json.dumps(line))
 
 
