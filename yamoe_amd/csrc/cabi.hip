@@ -88,6 +88,10 @@ int gemm_async_dgrad(const void *, const int *, int, const void *, void *, const
 template <typename T>
 int gemm_async_wgrad(const void *, const void *, void *, const int *, const int *, int, int, int, int, hipStream_t);
 bool gemm_async_supported(int Kd, int Nd, int lda, int ldb, long long a_span_bytes);
+bool gemm_f32_supported(int Kd, int Nd, int lda, int ldb, long long a_span_bytes);
+int gemm_f32_gate_up(const void *, const int *, const void *, const void *, void *, void *, const void *, int, int, int,
+                     int, int, hipStream_t);
+int gemm_f32_down(const void *, const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);
 bool wgrad_async_supported(int Md, int Nd);
 
 template <typename T> struct HasStreamPath { static constexpr bool value = sizeof(T) == 2; };
@@ -103,6 +107,9 @@ static int tiles_gate_up(const void *x, const int *sorted_idx, const void *w, co
     // the gathered source rows span the whole hidden_states tensor: N / K tokens of H elements
     if (gemm_async_supported(H, 2 * I, H, 2 * I, (long long)(N / K) * H * (long long)sizeof(T)))
       return gemm_async_gate_up<T>(x, sorted_idx, w, bias, act, pre, sched, N, K, E, H, I, small_rows, stream);
+  } else {
+    if (gemm_f32_supported(H, 2 * I, H, 2 * I, (long long)(N / K) * H * (long long)sizeof(T)))
+      return gemm_f32_gate_up(x, sorted_idx, w, bias, act, pre, sched, N, K, E, H, I, stream);
   }
   return gemm_gate_up<T>(x, sorted_idx, w, bias, act, pre, sched, N, K, E, H, I, stream);
 }
@@ -112,6 +119,8 @@ static int tiles_down(const void *act, const void *w, const void *bias, void *y,
   if constexpr (sizeof(T) == 2) {
     if (gemm_async_supported(I, H, I, H, 0))
       return gemm_async_down<T>(act, w, bias, y, sched, N, E, H, I, small_rows, stream);
+  } else {
+    if (gemm_f32_supported(I, H, I, H, 0)) return gemm_f32_down(act, w, bias, y, sched, N, E, H, I, stream);
   }
   return gemm_down<T>(act, w, bias, y, sched, N, E, H, I, stream);
 }

@@ -89,6 +89,14 @@ __device__ inline void glu_backward(float G, float U, float dh, float &dG, float
   dG = (G > kGluLimit) ? 0.0f : dgl * (s + g * s * (1.0f - s) * kGluAlpha);
 }
 
+// 16 bytes per lane from global memory straight into LDS at lds_base + lane * 16.
+__device__ inline void copy16_to_lds(const void *uniform_base, uint32_t lane_byte_off, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(lane_byte_off), "s"(uniform_base), "s"(lds_base)
+               : "memory", "m0");
+}
+
 // ---- schedule: device-built work lists shared by the expert GEMM kernels ---------------------
 // Layout of the schedule region (int32 words):
 //   [0] n_row_tiles   number of (expert, row-block) entries for the MFMA kernels

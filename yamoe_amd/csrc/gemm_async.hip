@@ -90,14 +90,6 @@ template <> struct Mma<f16_t> {
   }
 };
 
-// 16 bytes per lane from global memory straight into LDS at lds_base + lane * 16.
-__device__ inline void copy16_to_lds(const void *uniform_base, uint32_t lane_byte_off, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
-               :
-               : "v"(lane_byte_off), "s"(uniform_base), "s"(lds_base)
-               : "memory", "m0");
-}
-
 // two fp32 values rounded to T, packed low / high
 template <typename T> __device__ inline uint32_t pack2(float lo, float hi) {
   typedef T T2 __attribute__((ext_vector_type(2)));
