@@ -13,15 +13,20 @@ formula under test):
   route                 brute-force O(N^2) rank count on small inputs, numpy stable argsort,
                         permutation / monotonicity / stability invariants
   glu                   hand-computed known answers (tests/golden/glu_kat.json, made with Python's
-                        math module in tests/golden/make_glu_kat.py), limits G=0, U=-1, saturation
+                        math module in tests/golden/make_glu_kat.py), limits G=0, U=-1, saturation;
+                        bit-equal to transformers' GptOssExperts._apply_gate on random data
+                        (tests/test_oracle_vs_transformers.py)
   experts_loop          agrees with experts_dense (an independent formulation: all experts on all
                         tokens, dense weights) in fp64; special cases that reduce to one matmul
                         (single expert), to a row copy (interleaved-identity weights), to a
-                        bias-only closed form (zero weights), and linearity in routing weights
+                        bias-only closed form (zero weights), and linearity in routing weights;
+                        equal to transformers' GptOssExperts.forward in fp64 (an implementation from outside
+                        this repository, per-slot [T,K] routing weights)
   experts_capacity      brute-force per-slot Python loops on tiny inputs; equals experts_loop when
                         capacity >= max load
   experts_backward      torch.autograd.gradcheck of experts_capacity in fp64 (finite differences),
-                        and agreement between autograd and the closed-form experts_backward_closed
+                        agreement between autograd and the closed-form experts_backward_closed, and
+                        agreement of both with autograd through transformers' GptOssExperts
   sort_pairs            numpy's stable argsort on the masked key (a library routine), order and
                         stability invariants, two's-complement cases worked by hand
   bincount_cumsum       numpy bincount + cumsum (library), last entry = number of in-range items
@@ -35,8 +40,11 @@ formula under test):
                         (a library routine; values agree whatever its tie order), rows of scores sum to 1 and
                         are zero off the selection
 The reference ships no golden vectors or known-answer tests for this path (its tests directory is
-git-ignored), so no reference-held fixture exists to check against; no function here is
-"parity unpinned" in the sense of lacking an independent check.
+git-ignored), so no reference-held fixture exists to check against: every function here is pinned by
+independent checks, but agreement with the outputs of the reference's own CUDA op is unpinned.  Where
+the reference leaves a choice open this oracle fixes it: equal router logits pick the lower expert id
+(torch.topk's order among ties is unspecified), a [T,E] routing tensor with E == K is read as dense, and
+the routing gradient is placed once at [token, expert] (the reference's kernel permutes it twice).
 """
 import numpy as np
 import torch
