@@ -25,8 +25,10 @@ extern "C" {
 
 #define YAMOE_ABI_VERSION 1
 
-/* element type of activations, weights, biases and routing weights */
-enum { YAMOE_F32 = 0, YAMOE_F16 = 1, YAMOE_BF16 = 2 };
+/* element type of activations, weights, biases and routing weights.  YAMOE_F64 is taken by the row movers among
+ * the helper ops only (yamoe_padded_gather, yamoe_padded_scatter, yamoe_index_select), which the reference
+ * dispatches over double too (csrc/gather.cu:89, csrc/scatter.cu:128); everything else answers YAMOE_E_DTYPE. */
+enum { YAMOE_F32 = 0, YAMOE_F16 = 1, YAMOE_BF16 = 2, YAMOE_F64 = 3 };
 
 enum {
   YAMOE_E_ARG = -1,       /* bad size / null pointer / unsupported shape */

@@ -106,3 +106,43 @@ def test_yamoe_layer_forward(gpu, dtype):
     tol = REL_L2_TOL[dtype]
     assert report("layer", out.reshape(-1, H).double(), want, tol) < tol
     assert (scores != 0).sum(-1).max() <= K
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_yamoe_layer_reference_capacity_and_timing(gpu, dtype):
+    """expert_capacity = "reference" is the rule of torch-ext/yamoe/layers.py:161, ceil(tokens * top_k / experts): with
+    a skewed router every expert loaded above the mean loses its overflow, as the capacity oracle says; and the stage
+    timing of layers.py:118-122, 200-216 fills the same four keys."""
+    import yamoe_amd
+    B, S, H, I, E, K = 2, 160, 128, 64, 8, 2
+    blk = Block(H, I, E, K, dtype, 14)
+    with torch.no_grad():
+        blk.router.bias.copy_(torch.linspace(2.0, -2.0, E).to(dtype))    # the first experts are picked far more often
+    x = torch.randn(B, S, H, generator=torch.Generator().manual_seed(15)).to(dtype)
+    dev = Block(H, I, E, K, dtype, 14).to(gpu)
+    with torch.no_grad():
+        dev.router.bias.copy_(blk.router.bias)
+    dev.expert_capacity = "reference"
+    dev._timing_enabled = True
+    with torch.no_grad():
+        out, scores = yamoe_amd.Yamoe.forward(dev, x.to(gpu))
+    torch.cuda.synchronize()
+    out, scores = out.cpu(), scores.cpu()
+    assert set(dev._timing_stats) == {"router", "topk_softmax", "experts_kernel", "total"}
+    assert dev._timing_stats["total"] >= dev._timing_stats["experts_kernel"] > 0
+    cap = (B * S * K + E - 1) // E
+    idx = torch.topk(scores.float(), K, dim=-1).indices
+    counts = np.bincount(idx.numpy().ravel(), minlength=E)
+    assert counts.max() > cap, "the routing must overflow an expert for this test to mean anything"
+    args = (x.reshape(-1, H), idx, scores, blk.experts.gate_up_proj.data, blk.experts.gate_up_proj_bias.data,
+            blk.experts.down_proj.data, blk.experts.down_proj_bias.data)
+    want = O.experts_capacity(*args, cap, compute_dtype=torch.float64)
+    tol = REL_L2_TOL[dtype]
+    assert report("layer, reference capacity", out.reshape(-1, H).double(), want, tol) < tol
+    full = O.experts_capacity(*args, B * S, compute_dtype=torch.float64)
+    assert O.rel_l2(want, full) > 0.05        # and dropping changes the answer
+    dev.expert_capacity = None
+    dev._timing_enabled = False
+    with torch.no_grad():
+        out2, _ = yamoe_amd.Yamoe.forward(dev, x.to(gpu))
+    assert report("layer, no drop", out2.cpu().reshape(-1, H).double(), full, tol) < tol

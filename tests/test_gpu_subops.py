@@ -79,7 +79,7 @@ def routed(T, E, K, seed, skew=True):
     return ids, pos, bins
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.float64])
 @pytest.mark.parametrize("T,H,E,C,K", [(64, 128, 8, 4, 2), (300, 2880, 32, 50, 4), (17, 36, 3, 40, 1), (128, 130, 4, 0, 2)])
 def test_padded_gather_bit_exact(gpu, dtype, T, H, E, C, K):
     import yamoe_amd
@@ -95,7 +95,7 @@ def test_padded_gather_bit_exact(gpu, dtype, T, H, E, C, K):
         yamoe_amd.gather(x.to(gpu), torch.from_numpy(pos).to(gpu), torch.from_numpy(bins).to(gpu), out, E, C + 1, K)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.float64])
 @pytest.mark.parametrize("T,H,E,C,K,weighted", [(64, 128, 8, 4, 2, True), (300, 2880, 32, 50, 4, True),
                                                 (17, 36, 3, 40, 1, False), (90, 130, 4, 1000, 3, True)])
 def test_padded_scatter(gpu, dtype, T, H, E, C, K, weighted):
@@ -114,7 +114,7 @@ def test_padded_scatter(gpu, dtype, T, H, E, C, K, weighted):
     assert report("scatter", y.cpu().double(), want, REL_L2_TOL[dtype]) < REL_L2_TOL[dtype]
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.float64])
 def test_index_select_out(gpu, dtype):
     import yamoe_amd
     g = torch.Generator().manual_seed(2)

@@ -202,6 +202,27 @@ def experts_forward(hidden, router_indices, routing_weights, gate_up_proj, gate_
     return out
 
 
+def experts_backward(grad_out, hidden, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
+                     down_proj_bias, capacity, workspace=None, outs=None):
+    """yamoe_experts_backward through ctypes: returns (d_hidden, d_routing, d_gate_up_proj, d_gate_up_proj_bias,
+    d_down_proj, d_down_proj_bias); `workspace` (uint8 tensor) and the six outputs may be preallocated."""
+    _need_gpu(grad_out, hidden, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj, down_proj_bias)
+    p = problem(hidden, router_indices, routing_weights, gate_up_proj, capacity)
+    need = lib().yamoe_experts_backward_workspace_bytes(ctypes.byref(p))
+    if need == 0:
+        raise RuntimeError(lib().yamoe_last_error().decode())
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=hidden.device)
+    if outs is None:
+        outs = tuple(torch.empty_like(t) for t in (hidden, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
+                                                   down_proj_bias))
+    _check(lib().yamoe_experts_backward(ctypes.byref(p), _p(grad_out), _p(hidden), _p(router_indices), _p(routing_weights),
+                                        _p(gate_up_proj), _p(gate_up_proj_bias), _p(down_proj), _p(down_proj_bias),
+                                        *[_p(t) for t in outs], _p(workspace), workspace.numel(), _stream()),
+           "yamoe_experts_backward")
+    return outs
+
+
 STATIC_SCRATCH_BYTES = 32 << 20  # YAMOE_STATIC_SCRATCH_BYTES of include/yamoe_hip.h
 
 

@@ -33,23 +33,42 @@ template <typename T> struct ElemTraits;
 template <> struct ElemTraits<float> {
   static constexpr int kDtype = YAMOE_F32;
   static constexpr int kVec = 4;  // elements per 16-byte chunk
+  typedef float acc_t;
+  __device__ static inline float to_acc(float v) { return v; }
+  __device__ static inline float from_acc(float v) { return v; }
   __device__ static inline float to_f32(float v) { return v; }
   __device__ static inline float from_f32(float v) { return v; }
+};
+// double appears only in the helper ops that move rows (gather, scatter, index_select), which the reference
+// dispatches over double as well (csrc/gather.cu:89, csrc/scatter.cu:128); sums of doubles stay in double
+template <> struct ElemTraits<double> {
+  static constexpr int kDtype = YAMOE_F64;
+  static constexpr int kVec = 2;
+  typedef double acc_t;
+  __device__ static inline double to_acc(double v) { return v; }
+  __device__ static inline double from_acc(double v) { return v; }
+  __device__ static inline double from_f32(float v) { return (double)v; }
 };
 template <> struct ElemTraits<bf16_t> {
   static constexpr int kDtype = YAMOE_BF16;
   static constexpr int kVec = 8;
+  typedef float acc_t;
+  __device__ static inline float to_acc(bf16_t v) { return (float)v; }
+  __device__ static inline bf16_t from_acc(float v) { return (bf16_t)v; }
   __device__ static inline float to_f32(bf16_t v) { return (float)v; }
   __device__ static inline bf16_t from_f32(float v) { return (bf16_t)v; }
 };
 template <> struct ElemTraits<f16_t> {
   static constexpr int kDtype = YAMOE_F16;
   static constexpr int kVec = 8;
+  typedef float acc_t;
+  __device__ static inline float to_acc(f16_t v) { return (float)v; }
+  __device__ static inline f16_t from_acc(float v) { return (f16_t)v; }
   __device__ static inline float to_f32(f16_t v) { return (float)v; }
   __device__ static inline f16_t from_f32(float v) { return (f16_t)v; }
 };
 
-__host__ __device__ inline size_t dtype_size(int dtype) { return dtype == YAMOE_F32 ? 4 : 2; }
+__host__ __device__ inline size_t dtype_size(int dtype) { return dtype == YAMOE_F64 ? 8 : dtype == YAMOE_F32 ? 4 : 2; }
 
 __host__ __device__ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 

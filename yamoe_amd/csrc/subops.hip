@@ -235,16 +235,17 @@ __global__ __launch_bounds__(256) void padded_scatter_kernel(const T *src, const
   const int lane = threadIdx.x & 63;
   for (int t = blockIdx.x * 4 + (threadIdx.x >> 6); t < Tn; t += gridDim.x * 4) {
     for (int c = lane; c < H; c += 64) {
-      float acc = ElemTraits<T>::to_f32(y[(long long)t * H + c]);
+      typedef typename ElemTraits<T>::acc_t acc_t;
+      acc_t acc = ElemTraits<T>::to_acc(y[(long long)t * H + c]);
       for (int k = 0; k < top_k; ++k) {
         int row = slot_row[t * top_k + k];
         if (row < 0) continue;
         int e = row / C, i = row - e * C;
         int start = e == 0 ? 0 : bins[e - 1];
-        float w = weights ? ElemTraits<T>::to_f32(weights[start + i]) : 1.0f;
-        acc += w * ElemTraits<T>::to_f32(src[(long long)row * H + c]);
+        acc_t w = weights ? ElemTraits<T>::to_acc(weights[start + i]) : (acc_t)1;
+        acc += w * ElemTraits<T>::to_acc(src[(long long)row * H + c]);
       }
-      y[(long long)t * H + c] = ElemTraits<T>::from_f32(acc);
+      y[(long long)t * H + c] = ElemTraits<T>::from_acc(acc);
     }
   }
 }
@@ -313,6 +314,7 @@ extern "C" int yamoe_bincount_cumsum(const int32_t *input, int32_t n, int32_t *o
     case YAMOE_F32: { typedef float T; CALL; break; }                     \
     case YAMOE_BF16: { typedef bf16_t T; CALL; break; }                   \
     case YAMOE_F16: { typedef f16_t T; CALL; break; }                     \
+    case YAMOE_F64: { typedef double T; CALL; break; }                    \
     default: set_error("unknown dtype %d", dtype); return YAMOE_E_DTYPE;  \
   }
 

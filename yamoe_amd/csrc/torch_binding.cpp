@@ -28,6 +28,12 @@ int dtype_code(const at::Tensor &t, const char *name) {
   return -1;
 }
 
+// the row movers among the helper ops also take float64, like the reference's (csrc/gather.cu:89, csrc/scatter.cu:128)
+int mover_dtype_code(const at::Tensor &t, const char *name) {
+  if (t.scalar_type() == at::kDouble) return YAMOE_F64;
+  return dtype_code(t, name);
+}
+
 void check_rc(int rc, const char *what) {
   TORCH_CHECK(rc == 0, what, " failed (", rc, "): ", yamoe_last_error());
 }
@@ -175,7 +181,7 @@ void gather_op(const at::Tensor &x, const at::Tensor &indices, const at::Tensor 
   TORCH_CHECK(bins.numel() >= E, "bins must have at least E entries");
   const c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
   check_rc(yamoe_padded_gather(x.data_ptr(), indices.data_ptr<int>(), bins.data_ptr<int>(), output.data_ptr(), (int)T,
-                               (int)H, (int)E, (int)C, (int)top_k, dtype_code(x, "x"), current_stream()),
+                               (int)H, (int)E, (int)C, (int)top_k, mover_dtype_code(x, "x"), current_stream()),
            "yamoe_padded_gather");
 }
 
@@ -199,7 +205,7 @@ void scatter_op(const at::Tensor &src, const at::Tensor &indices, const at::Tens
   size_t ws_bytes = yamoe_padded_scatter_workspace_bytes((int)(T * top_k));
   at::Tensor ws = at::empty({(int64_t)ws_bytes}, src.options().dtype(at::kByte));
   check_rc(yamoe_padded_scatter(src.data_ptr(), indices.data_ptr<int>(), bins.data_ptr<int>(), w, y.data_ptr(), (int)T,
-                                (int)H, (int)E, (int)C, (int)top_k, dtype_code(src, "src"), ws.data_ptr(), ws_bytes,
+                                (int)H, (int)E, (int)C, (int)top_k, mover_dtype_code(src, "src"), ws.data_ptr(), ws_bytes,
                                 current_stream()),
            "yamoe_padded_scatter");
 }
@@ -242,7 +248,7 @@ at::Tensor index_select_out_op(at::Tensor out, at::Tensor in, at::Tensor idx_int
   TORCH_CHECK(out.scalar_type() == in.scalar_type() && out.numel() >= idx_int32.numel(), "out must match input's dtype and idx's length");
   const c10::hip::HIPGuardMasqueradingAsCUDA guard(in.device());
   check_rc(yamoe_index_select(in.data_ptr(), idx_int32.data_ptr<int>(), out.data_ptr(), idx_int32.numel(),
-                              dtype_code(in, "input"), current_stream()),
+                              mover_dtype_code(in, "input"), current_stream()),
            "yamoe_index_select");
   return out;
 }

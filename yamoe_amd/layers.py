@@ -1,6 +1,8 @@
 """Autograd glue for the `experts` op, mirroring `_ExpertsFn` of drbh/yamoe
 (torch-ext/yamoe/layers.py:6-100): same saved tensors, same order and arity of returned gradients.
 """
+import time
+
 import torch
 
 from ._ops import ops
@@ -48,8 +50,17 @@ class Yamoe(torch.nn.Module):
     """Drop-in `forward` for a GPT-OSS MLP block (router + experts), the role of `Yamoe.forward` in
     drbh/yamoe (torch-ext/yamoe/layers.py:106-218).  The host module provides `self.router`
     (weight [E,H], bias [E]) and `self.experts` (gate_up_proj, gate_up_proj_bias, down_proj,
-    down_proj_bias).  Unlike the reference, no assignment is dropped (capacity = tokens) and the
-    router gradient is kept when `enable_router_grads` is set.
+    down_proj_bias).  Attributes read if present:
+
+      num_experts, top_k     as in the reference (defaults 32 and 4)
+      enable_router_grads    kept as the host set it (the reference resets it on every call, layers.py:110)
+      expert_capacity        None (default): no assignment is dropped (capacity = tokens);
+                             "reference": the reference's rule ceil(tokens * top_k / num_experts) (layers.py:161),
+                             which drops the overflow of every expert loaded above the mean; or an int
+      _timing_enabled        stage times in ms into self._timing_stats (router, topk_softmax, experts_kernel,
+                             total), each closed by a device synchronisation as in layers.py:118-122, 200-216.
+                             The fused router kernel does the first two stages in one launch: its time is
+                             reported under "router" and "topk_softmax" is 0.
     """
 
     can_torch_compile: bool = False
@@ -58,22 +69,47 @@ class Yamoe(torch.nn.Module):
         batch, seq, hidden = hidden_states.shape
         num_experts = getattr(self, "num_experts", 32)
         top_k = getattr(self, "top_k", 4)
+        timing = getattr(self, "_timing_enabled", False)
+        stats = {}
+
+        def lap(name, since):
+            torch.cuda.synchronize()
+            now = time.perf_counter()
+            stats[name] = (now - since) * 1000
+            return now
+
+        if timing:
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
         x_flat = hidden_states.reshape(-1, hidden)
         want_router_grads = torch.is_grad_enabled() and getattr(self, "enable_router_grads", False)
         if router_kernel_takes(x_flat, self.router.weight, top_k) and not want_router_grads:
             # linear + top-k + softmax + dense scatter in one kernel
             router_indices, router_scores = ops.router_topk(x_flat, self.router.weight, self.router.bias, top_k)
+            if timing:
+                t1 = lap("router", t0)
+                stats["topk_softmax"] = 0.0
         else:
             # the same four steps as torch ops on the GPU (fp32 activations, shapes the kernel does not take, or a
             # router that is being trained: autograd needs the chain)
             logits = torch.nn.functional.linear(x_flat, self.router.weight, self.router.bias)
+            if timing:
+                t1 = lap("router", t0)
             top_vals, router_indices = torch.topk(logits, top_k, dim=-1)
             top_w = torch.nn.functional.softmax(top_vals, dim=-1, dtype=top_vals.dtype)
             router_scores = torch.zeros_like(logits).scatter_(1, router_indices, top_w)
+            if timing:
+                t1 = lap("topk_softmax", t1)
         I = self.experts.down_proj.shape[1]
         gate_up = self.experts.gate_up_proj[:, :, : 2 * I].contiguous()
         gate_up_bias = self.experts.gate_up_proj_bias[:, : 2 * I].contiguous()
-        capacity = x_flat.shape[0]
+        tokens = x_flat.shape[0]
+        capacity = getattr(self, "expert_capacity", None)
+        if capacity is None:
+            capacity = tokens
+        elif capacity == "reference":
+            capacity = (tokens * top_k + num_experts - 1) // num_experts
+        capacity = int(capacity)
         if want_router_grads:
             out = experts_autograd(x_flat, router_indices, router_scores, gate_up, gate_up_bias,
                                    self.experts.down_proj, self.experts.down_proj_bias, capacity, num_experts, top_k,
@@ -82,4 +118,8 @@ class Yamoe(torch.nn.Module):
             with torch.no_grad():
                 out = ops.experts(x_flat, router_indices, router_scores, gate_up, gate_up_bias,
                                   self.experts.down_proj, self.experts.down_proj_bias, capacity, num_experts, top_k)
+        if timing:
+            lap("experts_kernel", t1)
+            lap("total", t0)
+            self._timing_stats = stats
         return out.view(batch, seq, hidden), router_scores
