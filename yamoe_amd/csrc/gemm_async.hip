@@ -446,17 +446,35 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
   };
 
   if (has_bias) *(T *)(lds + kBiasOff + tid * 2) = bias_reg;  // (outside the ring and the staging area)
+  __syncthreads();  // every wave has finished reading the slab ring
   if constexpr (EPI == EPI_STORE && BNK) {
     // Row dots of the product with a second tensor of the output's shape, taken from the fp32 accumulators before they
     // are rounded (the routing gradient <grad_out . W_down^T, act>, csrc/experts_backward.cu:83-88): every wave writes
     // one partial sum per valid row, over its 128 columns of the tile; whoever reads them adds 2 * n_col_tiles values
-    // per row in a fixed order.
+    // per row in a fixed order.  The tile of the second tensor comes in through LDS by asynchronous copies, all in
+    // flight at once (the ring is dead): 512-byte rows, the 16-byte pieces of row r XOR-swizzled with r & 31 on the
+    // global side, so that the 32 lanes that read the same columns of 32 consecutive rows touch every bank once.
     if (args.dot_part != nullptr) {
+      {
+        const uint32_t lds_tile = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds);
+        const char *src = (const char *)((const T *)args.dot_with + out_row0 * args.ldc + n0);
+        const long long ld_bytes = (long long)args.ldc * (long long)sizeof(T);
+#pragma unroll 8
+        for (int i = 0; i < 32; ++i) {
+          const int row = 64 * wave + 2 * i + (lane >> 5);
+          int piece = (lane & 31) ^ (row & 31);
+          if (n0 + piece * 8 >= args.Nd) piece = 0;  // columns past the end: re-read valid ones, never used
+          const uint32_t off = (uint32_t)(min(row, rows_valid - 1) * ld_bytes + piece * 16);
+          copy16_to_lds(src, off, lds_tile + (uint32_t)(64 * wave + 2 * i) * 512u);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+      __syncthreads();
       const int n_part = 2 * args.n_col_tiles, part_col = 2 * (n0 / kBN) + wn;
+      const char *lp = lds + (wm * 32 + rl) * 512 + g * 8;
 #pragma unroll
       for (int mi = 0; mi < NMI; ++mi) {
         const int r = (mi * 2 + wm) * 32 + rl;
-        const T *wp = (const T *)args.dot_with + (out_row0 + min(r, rows_valid - 1)) * args.ldc + n0 + wn * 32 + 4 * g;
         float part = 0.0f;
 #pragma unroll
         for (int ni = 0; ni < NNI; ++ni)
@@ -465,7 +483,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
             // a run of four columns is valid or invalid as a whole (the column count is a multiple of 8)
             if (n0 + (ni * 2 + wn) * 32 + 8 * q + 4 * g < args.Nd) {
               float w4[4];
-              load4_f32(wp + ni * 64 + 8 * q, w4);
+              load4_f32((const T *)(lp + mi * 64 * 512 + ((((ni * 2 + wn) * 4 + q) ^ rl) << 4)), w4);
 #pragma unroll
               for (int i = 0; i < 4; ++i) part += acc[mi][ni][4 * q + i] * w4[i];
             }
@@ -473,9 +491,9 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
         part += __shfl_xor(part, 32);
         if (g == 0 && r < rows_valid) args.dot_part[(out_row0 + r) * n_part + part_col] = part;
       }
+      __syncthreads();  // the staging area is about to be overwritten with the output tile
     }
   }
-  __syncthreads();  // every wave has finished reading the slab ring
   if constexpr (EPI == EPI_STORE) {
     stage_biased();
     __syncthreads();

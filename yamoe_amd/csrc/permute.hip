@@ -136,18 +136,32 @@ __global__ __launch_bounds__(kRowThreads) void combine_backward_kernel(
     T *o = g_y_perm + (size_t)p * H;
     float dot = 0.0f;
     constexpr int V = ElemTraits<T>::kVec;
-    if (H % V == 0) {  // 16 bytes per lane (rows are 16-byte aligned then)
-      for (int c = lane; c < H / V; c += kWave) {
-        u32x4 graw = ((const u32x4 *)g)[c], braw = ((const u32x4 *)bd)[c], oraw;
-        const T *gv = (const T *)&graw, *bv = (const T *)&braw;
-        T *ov = (T *)&oraw;
+    if (H % V == 0) {  // 16 bytes per lane (rows are 16-byte aligned then), four chunks of both rows in flight
+      const int n_chunks = H / V;
+      for (int c0 = lane; c0 < n_chunks; c0 += 4 * kWave) {
+        u32x4 graw[4], braw[4];
 #pragma unroll
-        for (int j = 0; j < V; ++j) {
-          float x = ElemTraits<T>::to_f32(gv[j]);
-          dot += x * ElemTraits<T>::to_f32(bv[j]);
-          ov[j] = ElemTraits<T>::from_f32(x * w);
+        for (int u = 0; u < 4; ++u) {
+          const int c = min(c0 + u * kWave, n_chunks - 1);
+          graw[u] = ((const u32x4 *)g)[c];
+          braw[u] = ((const u32x4 *)bd)[c];
         }
-        ((u32x4 *)o)[c] = oraw;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int c = c0 + u * kWave;
+          if (c < n_chunks) {
+            const T *gv = (const T *)&graw[u], *bv = (const T *)&braw[u];
+            u32x4 oraw;
+            T *ov = (T *)&oraw;
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+              float x = ElemTraits<T>::to_f32(gv[j]);
+              dot += x * ElemTraits<T>::to_f32(bv[j]);
+              ov[j] = ElemTraits<T>::from_f32(x * w);
+            }
+            ((u32x4 *)o)[c] = oraw;
+          }
+        }
       }
     } else {
       for (int c = lane; c < H; c += kWave) {
