@@ -130,7 +130,8 @@ int yamoe_experts_forward(const yamoe_problem *p, const void *hidden_states,
  * Same arguments, kernels and results as yamoe_experts_forward, but the workspace is an array of
  * YAMOE_STATIC_SCRATCH_BYTES that is part of the library's device image (each GPU the library runs
  * on holds its copy until the process ends).  The call allocates and frees nothing; its first call
- * on a device looks the array's address up (one hipGetSymbolAddress).  Problems whose
+ * on a device looks the array's address up (one hipGetSymbolAddress, which may load the device
+ * image: make that first call before a stream capture begins, not inside it).  Problems whose
  * yamoe_experts_workspace_bytes() exceeds the array are rejected with YAMOE_E_WORKSPACE (at
  * H = I = 2880 in a 16-bit dtype the limit is about 2900 (token, expert) assignments, e.g. 725
  * tokens at top-4).  All calls on one GPU share that GPU's array: two calls whose work overlaps on
