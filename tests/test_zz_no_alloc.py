@@ -57,3 +57,32 @@ def test_static_workspace_forward_refuses_large_problems(gpu):
     rc = _cabi.lib().yamoe_experts_forward_static(ctypes.byref(p), *([ptr] * 8), ptr, None)
     assert rc == -2, rc   # YAMOE_E_WORKSPACE
     assert b"built-in" in _cabi.lib().yamoe_last_error()
+
+
+def test_static_workspace_forward_in_a_hip_graph(gpu):
+    """The callers it is for: captured once (after a first eager call, which looks the array's address up), replayed
+    with other work in between, every replay equal to the eager result."""
+    from yamoe_amd import _cabi
+    d = make_inputs(500, 256, 128, 8, 2, torch.bfloat16, seed=55, w_std=0.05, bias_std=0.1, zipf=0.6)
+    g = [d[k].to(gpu) for k in KEYS]
+    want = _cabi.experts_forward(*g, 500)
+    out = torch.zeros_like(want)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        _cabi.experts_forward_static(*g, 500, out)            # first call on this device happens outside the capture
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        _cabi.experts_forward_static(*g, 500, out)
+    small = make_inputs(30, 256, 128, 8, 2, torch.bfloat16, seed=56, w_std=0.05, bias_std=0.1)
+    gs = [small[k].to(gpu) for k in KEYS]
+    for rep in range(3):
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), rep
+        scratch_user = torch.empty(30, 256, dtype=torch.bfloat16, device=gpu)
+        _cabi.experts_forward_static(*gs, 30, scratch_user)   # another problem on the same array between replays
+        torch.cuda.synchronize()
