@@ -97,8 +97,9 @@ def main():
                     help="only the headline workload and its dominant kernel (for profiler runs)")
     ap.add_argument("--only", default="", help="with --no-configs: also run this one of decode, zipf, readme, backward")
     ap.add_argument("--extras", action="store_true",
-                    help="also time the vendor library's dense GEMM on the two forward GEMM shapes, and the routing "
-                         "and permute kernels of the Zipf workload on their own")
+                    help="also time the vendor library's dense GEMM on the two forward GEMM shapes, the routing and "
+                         "permute kernels of the Zipf workload on their own, and the gate_up launch on zero weights "
+                         "(how much of its time is the power limit)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy kernel (a known FETCH_SIZE / WRITE_SIZE for counter runs)")
     args = ap.parse_args()
@@ -188,6 +189,22 @@ def main():
                     avg_launch_ms=round(gu_ms, 4),
                     down_gemm=dict(achieved=round(dn_tflops, 2), frac=round(dn_tflops / PEAK_BF16_TFLOPS, 4),
                                    avg_launch_ms=round(dn_ms, 4)))
+    data_dependence = None
+    if args.extras:
+        # the same gate_up launch on operands that do not toggle the datapath: how much of the time is the power limit
+        zero_w = torch.zeros_like(d["gate_up_proj"])
+
+        def gu_zero():
+            _cabi.lib().yamoe_gate_up(
+                _cabi._p(d["hidden"]), _cabi._p(si), _cabi._p(zero_w), _cabi._p(d["gate_up_proj_bias"]),
+                _cabi._p(act), None, _cabi._p(sched), n_rows, K, E, H, I, _cabi.BF16, _cabi._stream())
+        spin_up(gu_zero, args.spinup_ms)
+        z_ms = event_time_ms(gu_zero, args.steps)
+        spin_up(gu_launch, args.spinup_ms)
+        r_ms = event_time_ms(gu_launch, args.steps)
+        data_dependence = dict(gate_up_random_data_ms=round(r_ms, 4), gate_up_zero_weights_ms=round(z_ms, 4),
+                               tflops_zero_weights=round(gu_flop / (z_ms * 1e-3) / 1e12, 1))
+        del zero_w
     del act, y
 
     # ---------------- CPU baseline on the same batch, and the parity of the timed op ---------------------
@@ -275,7 +292,7 @@ def main():
         torch.cuda.empty_cache()
 
     # ---------------- cfg4: Zipf-skewed routing, 16384 tokens, 128 experts -----------------------------------
-    extras = {} if args.extras else None
+    extras = dict(gate_up_data_dependence=data_dependence) if args.extras else None
     if wanted("zipf"):
         zc = workloads.CONFIGS["zipf"]
         hostz, _ = workloads.make_config("zipf", seed=0, weights=False)
