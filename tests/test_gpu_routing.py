@@ -140,8 +140,9 @@ def test_schedule_lists(gpu, N, E, C, stream_rows):
     assert [tuple(t) for t in small.tolist()] == want_small
     # The cut table: 9 cuts that split the tile list into 8 shares of (nearly) equal cost for any number of
     # column tiles; every cut lies on an (expert, column tile) boundary and the cuts are monotone.
+    # cost weight of a tile: 3 + 2 per 64 rows; an expert with a single row tile weighs at least 8
     weight = lambda rows: 3 + 2 * ((rows + 63) // 64)
-    w_tiles = [weight(t[2]) for t in want_tiles]
+    w_tiles = [max(weight(t[2]), 8) if t[4] == 1 else weight(t[2]) for t in want_tiles]
     assert sched[4] == sum(w_tiles)
     for n_col in (1, 12, 23):
         cuts = []

@@ -122,7 +122,7 @@ __device__ inline void copy16_to_lds(const void *uniform_base, uint32_t lane_byt
 //   [1] n_small       number of experts on the weight-streaming path
 //   [2] n_active      experts with at least one kept row
 //   [3] n_kept        total kept rows
-//   [4] weight_total  sum of the row-tile cost weights (sched_tile_weight)
+//   [4] weight_total  sum of the experts' cost weights (sched_group_weight)
 //   [8 + 4x ...)      x = 0..8: where the tile list is cut so that each of the 8 XCDs gets the same share of
 //                     the cost: {first row tile of the expert the cut falls in, f, 0, row tiles of that
 //                     expert}, f = the cut's position inside that expert's tiles in 1/65536ths; in a GEMM
@@ -140,6 +140,15 @@ constexpr int kXcds = 8;
 // Relative cost of one row tile in the MFMA kernels: a fixed part (prologue, epilogue, copies of the weight
 // slabs) plus one part per 64 rows (the MFMA blocks of the slower wave row).
 __host__ __device__ inline int sched_tile_weight(int rows) { return 3 + 2 * ((rows + 63) / 64); }
+// An expert with a single row tile shares its weight slabs with nobody: every one of its column tiles pulls them from
+// HBM at one workgroup's latency-bound rate, which takes about as long as a tile of 150-200 rows however few rows it
+// has (measured on the Zipf-skewed workload: 2 % of the step between this floor and none).
+constexpr int kLoneTileWeight = 8;
+__host__ __device__ inline int sched_group_weight(int tiles, int per_tile, int kept) {
+  if (tiles <= 0) return 0;
+  int w = (tiles - 1) * sched_tile_weight(per_tile) + sched_tile_weight(kept - (tiles - 1) * per_tile);
+  return tiles == 1 && w < kLoneTileWeight ? kLoneTileWeight : w;
+}
 // flat tile index of cut x of the schedule for a GEMM with n_col_tiles column tiles
 __host__ __device__ inline int sched_cut(const int *sched, int x, int n_col_tiles) {
   const int *c = sched + kSchedCuts + 4 * x;

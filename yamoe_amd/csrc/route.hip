@@ -189,7 +189,7 @@ __device__ inline void build_schedule_wave(const int *counts, const int *offsets
       int is_small = kept > 0 && kept <= stream_max_rows;
       int tiles = (kept > 0 && !is_small) ? ceil_div(kept, kRowTile) : 0;
       int per_tile = tiles > 0 ? min(kRowTile, (ceil_div(kept, tiles) + 31) & ~31) : 0;
-      int w = tiles > 0 ? (tiles - 1) * sched_tile_weight(per_tile) + sched_tile_weight(kept - (tiles - 1) * per_tile) : 0;
+      int w = sched_group_weight(tiles, per_tile, kept);
       int tot_w, tot_t;
       int w_pre = w_before + wave_exclusive_scan(w, lane, tot_w);
       int t_pre = t_before + wave_exclusive_scan(tiles, lane, tot_t);
