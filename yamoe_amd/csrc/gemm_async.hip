@@ -807,7 +807,80 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
     __syncthreads();
     read_frags(0, 0, fa0, fb0);
   }
-  auto slab_step = [&](int s, auto cfg) {
+  // In the pipelined loop the ring stage of every slab is a compile-time constant (the loop is unrolled by the ring
+  // depth), so that an operand read is one ds_read with an immediate offset from a per-lane base and a copy's LDS
+  // address one scalar add: with the stage computed per slab (a division by 3, then one vector add per read) the
+  // loop carried 3.4 vector instructions per MFMA, 30 of them in a block ahead of each slab's first MFMA.
+  const char *pa[NACC], *pb[4];
+#pragma unroll
+  for (int mi = 0; mi < NACC; ++mi) pa[mi] = lds + a_rd[mi];
+#pragma unroll
+  for (int ni = 0; ni < 4; ++ni) pb[ni] = lds + kSmallBRing + b_rd[ni];
+  const uint32_t lds_a_wave = lds0 + (uint32_t)(8 * wave) * 256u, lds_b_wave = lds0 + kSmallBRing + (uint32_t)(8 * wave) * 512u;
+  auto read_frag_c = [&](auto stage, int ks, int f, u32x4 (&fa)[NACC], u32x4 (&fb)[4]) {
+    constexpr int ST = decltype(stage)::value;
+    const bool is_a = f == 1 || f >= 5;
+    const int idx = is_a ? (f == 1 ? 0 : f - 4) : (f == 0 ? 0 : f - 1);
+    const char *sp = is_a ? pa[idx] + ST * kSmallAStage + ks * 4096 : pb[idx] + ST * kSmallBStage + ks * 8192;
+    u32x2 lo = lds_read_tr16(sp);
+    u32x2 hi = lds_read_tr16(sp + (is_a ? 1024 : 2048));
+    u32x4 v = (u32x4){lo[0], lo[1], hi[0], hi[1]};
+    if (is_a) fa[idx] = v; else fb[idx] = v;
+  };
+  auto copy_a_c = [&](auto stage, int slab, int i) {
+    constexpr int ST = decltype(stage)::value;
+    copy16_to_lds(a_base + (long long)slab * kBK * lda_bytes, a_off[i], lds_a_wave + (uint32_t)(ST * kSmallAStage + 4 * i * 256));
+  };
+  auto copy_b_c = [&](auto stage, int slab, int i) {
+    constexpr int ST = decltype(stage)::value;
+    copy16_to_lds(b_base + (long long)slab * kBK * ldb_bytes, b_off[i], lds_b_wave + (uint32_t)(ST * kSmallBStage + 2 * i * 512));
+  };
+  // slab s sits in ring stage ST
+  auto slab_step = [&](int s, auto cfg, auto stage) {
+    typedef decltype(cfg) C;
+    constexpr int ST = decltype(stage)::value;
+    typedef std::integral_constant<int, (ST + 1) % kSmallStages> Next;   // slab s + 1
+    typedef std::integral_constant<int, (ST + 2) % kSmallStages> Next2;  // slab s + 2; slab s + 3 takes stage ST again
+    __builtin_amdgcn_sched_barrier(0);
+    {
+      constexpr int kC = C::P1 ? 3 : 0, kItems = kC + kFrags;
+#pragma unroll
+      for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
+        if (j < kMma) Mma<T>::run(fb0[j & 3], fa0[j >> 2], acc[j >> 2][j & 3]);
+        if (j < kSlots) {
+#pragma unroll
+          for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
+            if (i < kC) { if (i == 0) copy_a_c(Next2(), s + 2, 1); else copy_b_c(Next2(), s + 2, 1 + i); }
+            else read_frag_c(stage, 1, i - kC, fa1, fb1);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    if constexpr (C::VM == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+    else if constexpr (C::VM == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if constexpr (C::ZERO) zero_tail(s + 1);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    {
+      constexpr int kC = C::P2 ? 3 : 0, kItems = kC + (C::NEXT ? kFrags : 0);
+#pragma unroll
+      for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
+        if (j < kMma) Mma<T>::run(fb1[j & 3], fa1[j >> 2], acc[j >> 2][j & 3]);
+        if (j < kSlots) {
+#pragma unroll
+          for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
+            if (i < kC) { if (i == 0) copy_a_c(stage, s + 3, 0); else copy_b_c(stage, s + 3, i - 1); }
+            else read_frag_c(Next(), 0, i - kC, fa0, fb0);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+  // the same step with the ring stage taken from the slab number at run time: for the slabs the unrolled loop leaves
+  // over and for the last three (the stage they start in depends on the slab count)
+  auto slab_step_rt = [&](int s, auto cfg) {
     typedef decltype(cfg) C;
     __builtin_amdgcn_sched_barrier(0);
     {
@@ -847,13 +920,22 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
     }
   };
   if (n_slabs >= 6) {
-    slab_step(0, WStepCfg<false, true, true, false, 6>());
+    typedef std::integral_constant<int, 0> S0;
+    typedef std::integral_constant<int, 1> S1;
+    typedef std::integral_constant<int, 2> S2;
+    typedef WStepCfg<true, true, true, false, 6> Steady;
+    slab_step(0, WStepCfg<false, true, true, false, 6>(), S0());
     int s = 1;
-    for (; s + 3 < n_slabs; ++s) slab_step(s, WStepCfg<true, true, true, false, 6>());
-    // s = n_slabs - 3
-    slab_step(s, WStepCfg<true, false, true, false, 6>());
-    slab_step(s + 1, WStepCfg<false, false, true, true, 0>());
-    slab_step(s + 2, WStepCfg<false, false, false, false, -1>());
+    for (; s + 5 < n_slabs; s += 3) {  // steady state, three slabs per round: stages 1, 2, 0
+      slab_step(s, Steady(), S1());
+      slab_step(s + 1, Steady(), S2());
+      slab_step(s + 2, Steady(), S0());
+    }
+    for (; s + 3 < n_slabs; ++s) slab_step_rt(s, Steady());  // at most two
+    // the last three slabs (s = n_slabs - 3): no new copies; the last slab's missing rows are zeroed
+    slab_step_rt(s, WStepCfg<true, false, true, false, 6>());
+    slab_step_rt(s + 1, WStepCfg<false, false, true, true, 0>());
+    slab_step_rt(s + 2, WStepCfg<false, false, false, false, -1>());
   } else {
     for (int s = 0; s < n_slabs; ++s) {
       if (kFrags > 0) read_frags(s, 1, fa1, fb1);
