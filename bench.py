@@ -288,11 +288,29 @@ def main():
             decode["parity"] = parity_of(dstep().float().cpu(), want, 1e-2, "fp32 oracle, all 64 tokens, device-drawn weights copied back")
         configs["cfg3_decode_bf16"] = dict(ms=round(d_ms, 4), gbs=round(gbs, 1), frac_of_peak=round(gbs / PEAK_HBM_GBS, 4),
                                            peak="HBM %.0f GB/s" % PEAK_HBM_GBS, parity=decode["parity"])
+        decode_batches = None
+        if args.extras:
+            # the same layer with the first 1, 2, 4, ... of the 64 tokens: few experts, little to hide latency behind
+            decode_batches = {}
+            for tb in (1, 2, 4, 8, 16, 32):
+                ab = [dd["hidden"][:tb].contiguous(), dd["router_indices"][:tb].contiguous(),
+                      dd["routing_weights"][:tb].contiguous()] + ad[3:]
+                act_b = int((np.bincount(hostd["router_indices"][:tb].numpy().ravel(), minlength=Ed) > 0).sum())
+                nb = workloads.algorithmic_bytes_decode(act_b, tb, Kd, Ed, H, I)
+
+                def bstep():
+                    return yamoe_amd.experts(*ab, tb, Ed, Kd)
+                spin_up(bstep, args.spinup_ms / 4)
+                b_ms = event_time_ms(bstep, args.steps)
+                decode_batches["tokens_%d" % tb] = dict(us=round(b_ms * 1e3, 1), active_experts=act_b,
+                                                        gbs=round(nb / (b_ms * 1e-3) / 1e9, 1))
         del dd, ad
         torch.cuda.empty_cache()
 
     # ---------------- cfg4: Zipf-skewed routing, 16384 tokens, 128 experts -----------------------------------
     extras = dict(gate_up_data_dependence=data_dependence) if args.extras else None
+    if args.extras and wanted("decode"):
+        extras["decode_small_batches"] = decode_batches
     if wanted("zipf"):
         zc = workloads.CONFIGS["zipf"]
         hostz, _ = workloads.make_config("zipf", seed=0, weights=False)

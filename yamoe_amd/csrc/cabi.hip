@@ -277,12 +277,15 @@ static int forward_impl(const yamoe_problem *p, const void *x, const void *idx, 
   const int stream_rows = HasStreamPath<T>::value ? kStreamMaxRows : 0;
   YAMOE_TRY(route_and_schedule(idx, p->idx_i64, N, p->E, p->capacity, b.sorted_expert, b.sorted_idx, b.counts, b.offsets,
                                b.inv_pos, b.route_ws, b.route_ws_bytes, stream_rows, b.schedule, b.schedule_bytes, st));
-  YAMOE_TRY(tiles_gate_up<T>(x, b.sorted_idx, wgu, bgu, b.act, nullptr, b.schedule, N, p->K, p->E, p->H, p->I, stream_rows,
-                             stream));
+  // with no more assignments than a streamed expert may have rows, every expert is streamed: the tile lists are empty
+  const bool tiles = N > stream_rows;
+  if (tiles)
+    YAMOE_TRY(tiles_gate_up<T>(x, b.sorted_idx, wgu, bgu, b.act, nullptr, b.schedule, N, p->K, p->E, p->H, p->I, stream_rows,
+                               stream));
   if constexpr (HasStreamPath<T>::value)
     YAMOE_TRY(stream_gate_up<T>(x, b.sorted_idx, wgu, bgu, b.act, nullptr, b.schedule, N, p->K, p->E, p->H, p->I,
                                 stream));
-  YAMOE_TRY(tiles_down<T>(b.act, wd, bd, b.y_perm, b.schedule, N, p->E, p->H, p->I, stream_rows, stream));
+  if (tiles) YAMOE_TRY(tiles_down<T>(b.act, wd, bd, b.y_perm, b.schedule, N, p->E, p->H, p->I, stream_rows, stream));
   if constexpr (HasStreamPath<T>::value)
     YAMOE_TRY(stream_down<T>(b.act, wd, bd, b.y_perm, b.schedule, N, p->E, p->H, p->I, stream));
   YAMOE_TRY(launch_combine<T>(b.y_perm, b.inv_pos, idx, p->idx_i64, rw, p->rw_cols, out, p->T, p->K, p->E, p->H,

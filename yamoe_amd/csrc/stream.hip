@@ -9,6 +9,12 @@
 // activations.  No LDS is touched until the final cross-wave reduction.  Two steps of loads are
 // kept in flight per wave, 8 waves per CU.
 //
+// A launch that can hold only a few experts (a handful of tokens: at most kStreamFewBlocks workgroups) has too few
+// workgroups to keep HBM busy that way: 4 experts x 23 slabs with two steps of 8 KB in flight per wave are 6 MB on
+// the way, where 8 TB/s x 2 us of latency want 16 MB.  Such a launch takes 8 waves per workgroup with three steps in
+// flight each instead (a workgroup per CU; 16 waves would leave a wave 128 registers, not enough for two steps), folded
+// into the first four before the same finish.
+//
 // The lane that holds accumulator column c of MFMA j owns output column 8c + j, so the 8
 // accumulators of a lane are 8 consecutive output columns: the interleaved (gate, up) pairs of the
 // clamped SwiGLU (csrc/moe.cpp:164-180) meet in one lane.
@@ -16,8 +22,9 @@
 
 namespace yamoe {
 
-constexpr int kStreamThreads = 256;
-constexpr int kStreamWaves = 4;
+constexpr int kStreamWaves = 4;        // waves that finish a slab; a workgroup has 4 or 8
+constexpr int kStreamManyWaves = 8;
+constexpr int kStreamFewBlocks = 1024;  // launches with fewer (expert, slab) workgroups than this take 8 waves each
 constexpr int kSlabCols = 128;
 
 typedef float f32x4v __attribute__((ext_vector_type(4)));
@@ -47,8 +54,8 @@ struct StreamArgs {
   int a_div, Kd, Nd, lda, ldc, n_slabs, N, E;
 };
 
-template <typename T, bool GLU, bool GATHER>
-__global__ __launch_bounds__(kStreamThreads, 2) void stream_gemm_kernel(const StreamArgs args) {
+template <typename T, bool GLU, bool GATHER, int WAVES, int DEPTH>
+__global__ __launch_bounds__(64 * WAVES, WAVES == kStreamWaves ? 2 : 1) void stream_gemm_kernel(const StreamArgs args) {
   __shared__ float red[kStreamWaves * 8 * 4 * kWave];  // [wave][j][v][lane]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const ScheduleView sv = schedule_view(args.sched, args.N, args.E);
@@ -74,7 +81,7 @@ __global__ __launch_bounds__(kStreamThreads, 2) void stream_gemm_kernel(const St
   for (int j = 0; j < 8; ++j) acc[j] = (f32x4v){0.f, 0.f, 0.f, 0.f};
 
   const int n_steps = (args.Kd + 31) / 32;
-  u32x4 bw0[8], bw1[8], aw0, aw1;
+  u32x4 bw[DEPTH][8], aw[DEPTH];
 
   auto fetch = [&](int step, u32x4 (&bw)[8], u32x4 &aw) {
     int k0 = step * 32;
@@ -100,25 +107,49 @@ __global__ __launch_bounds__(kStreamThreads, 2) void stream_gemm_kernel(const St
     }
   };
 
-  // steps wave, wave+4, ... ; two in flight
+  // steps wave, wave + WAVES, ... ; DEPTH in flight (the loop is unrolled by DEPTH, so the buffers are fixed registers)
   int step = wave;
-  if (step < n_steps) fetch(step, bw0, aw0);
-  while (step < n_steps) {
-    if (step + kStreamWaves < n_steps) fetch(step + kStreamWaves, bw1, aw1);
-    consume(bw0, aw0);
-    step += kStreamWaves;
-    if (step >= n_steps) break;
-    if (step + kStreamWaves < n_steps) fetch(step + kStreamWaves, bw0, aw0);
-    consume(bw1, aw1);
-    step += kStreamWaves;
+#pragma unroll
+  for (int d = 0; d < DEPTH - 1; ++d)
+    if (step + d * WAVES < n_steps) fetch(step + d * WAVES, bw[d], aw[d]);
+  for (bool more = step < n_steps; more;) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      if (more) {
+        if (step + (DEPTH - 1) * WAVES < n_steps) fetch(step + (DEPTH - 1) * WAVES, bw[(d + DEPTH - 1) % DEPTH], aw[(d + DEPTH - 1) % DEPTH]);
+        consume(bw[d], aw[d]);
+        step += WAVES;
+        more = step < n_steps;
+      }
+    }
   }
 
-  // ---- reduce the 4 partial sums and finish -----------------------------------------------------
+  // ---- reduce the partial sums and finish ---------------------------------------------------------
+  // more than four waves: waves 4r .. 4r+3 hand their sums to waves 0 .. 3, one group after the other (a fixed order)
+  for (int r = 1; r < WAVES / kStreamWaves; ++r) {
+    if (wave / kStreamWaves == r) {
 #pragma unroll
-  for (int j = 0; j < 8; ++j)
+      for (int j = 0; j < 8; ++j)
 #pragma unroll
-    for (int v = 0; v < 4; ++v) red[((wave * 8 + j) * 4 + v) * kWave + lane] = acc[j][v];
+        for (int v = 0; v < 4; ++v) red[(((wave - kStreamWaves * r) * 8 + j) * 4 + v) * kWave + lane] = acc[j][v];
+    }
+    __syncthreads();
+    if (wave < kStreamWaves) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[j][v] += red[((wave * 8 + j) * 4 + v) * kWave + lane];
+    }
+    __syncthreads();
+  }
+  if (wave < kStreamWaves) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) red[((wave * 8 + j) * 4 + v) * kWave + lane] = acc[j][v];
+  }
   __syncthreads();
+  if (wave >= kStreamWaves) return;  // (after the last workgroup barrier)
 
   // wave w finishes accumulator columns j = 2w, 2w+1 (one gate/up pair per lane)
   float sum[2][4];
@@ -164,7 +195,13 @@ template <typename T, bool GLU, bool GATHER>
 static int launch_stream(const StreamArgs &a, hipStream_t stream) {
   long long blocks = (long long)sched_max_small(a.N, a.E) * a.n_slabs;
   if (blocks <= 0) return 0;
-  hipLaunchKernelGGL((stream_gemm_kernel<T, GLU, GATHER>), dim3((unsigned)blocks), dim3(kStreamThreads), 0, stream, a);
+  if (blocks < kStreamFewBlocks) {
+    hipLaunchKernelGGL((stream_gemm_kernel<T, GLU, GATHER, kStreamManyWaves, 3>), dim3((unsigned)blocks),
+                       dim3(64 * kStreamManyWaves), 0, stream, a);
+  } else {
+    hipLaunchKernelGGL((stream_gemm_kernel<T, GLU, GATHER, kStreamWaves, 2>), dim3((unsigned)blocks), dim3(64 * kStreamWaves),
+                       0, stream, a);
+  }
   return check_launch("stream_gemm_kernel");
 }
 
