@@ -140,3 +140,56 @@ def test_backward_gptoss20b_full(gpu):
     grads = run_bwd(d, gy, c["T"], gpu)
     want = O.experts_backward(gy, *args(d), c["T"], compute_dtype=torch.float32)
     check(grads, want, torch.bfloat16, "gptoss20b")
+
+
+CLAMPED = [
+    # dtype, T, H, I, E, K, weight std: pre-activations of std 3 to 8, a good part of them beyond the clamp at 7
+    (torch.bfloat16, 700, 256, 128, 4, 2, 0.5),    # asynchronous-copy kernels
+    (torch.float16, 700, 256, 128, 4, 2, 0.5),
+    (torch.bfloat16, 64, 200, 72, 4, 2, 0.4),      # register-staged kernels (contraction not a multiple of 64)
+    (torch.bfloat16, 600, 2880, 512, 2, 1, 0.05),  # the GPT-OSS width, where sqrt(2880) * 0.05 does the same
+]
+
+
+@pytest.mark.parametrize("dtype,T,H,I,E,K,w_std", CLAMPED)
+def test_backward_pre_activations_near_the_clamp(gpu, dtype, T, H, I, E, K, w_std):
+    """The backward reads the pre-activations back in the activation dtype and tests them against the clamp limit
+    (csrc/experts_backward.cu:285-299).  A value just beyond the limit that rounds onto it (bf16: anything in
+    (7, 7.016]) must still count as clamped, as it does in the forward and in the oracle's fp32: with plain rounding
+    d_hidden and the gate_up gradients of these cases are off by 1.2e-2 to 5e-2, a few elements each wrong by its
+    whole size."""
+    print("backward_clamp", dtype, T, H, I, E, K, w_std, flush=True)
+    d = make_inputs(T, H, I, E, K, dtype, seed=T + H, w_std=w_std, bias_std=0.1)
+    gy = torch.randn(T, H, generator=torch.Generator().manual_seed(4)).to(dtype)
+    grads = run_bwd(d, gy, T, gpu)
+    want = O.experts_backward(gy, *args(d), T, compute_dtype=torch.float32)
+    check(grads, want, dtype, "clamp")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T", [300, 5])
+def test_stored_pre_activations_keep_the_clamp_decision(gpu, dtype, T):
+    """yamoe_gate_up's optional pre-activation output: |value| > 7 in fp32 is never stored as exactly 7 (tile kernels
+    for T = 300, streaming kernel for T = 5), values within the limit are the plain rounding."""
+    from yamoe_amd import _cabi
+    H, I, E, K = 128, 64, 4, 2
+    d = make_inputs(T, H, I, E, K, dtype, seed=31, w_std=0.6, bias_std=0.1)
+    g = to_dev(d, gpu)
+    se, si, counts, offsets, inv = _cabi.route(g["router_indices"], E, T)
+    sched = _cabi.build_schedule(counts, offsets, T * K, T, 16)
+    act, pre = _cabi.gate_up(g["hidden"], si, g["gate_up_proj"], g["gate_up_proj_bias"], sched, K, want_pre=True)
+    torch.cuda.synchronize()
+    tok = si.cpu().long() // K
+    e = d["router_indices"].reshape(-1)[si.cpu().long()]
+    x = d["hidden"].double()[tok]
+    want = torch.stack([x[p] @ d["gate_up_proj"][int(e[p])].double() + d["gate_up_proj_bias"][int(e[p])].double()
+                        for p in range(T * K)])
+    got = pre.cpu().double()
+    gate_w, up_w, gate_g, up_g = want[:, 0::2], want[:, 1::2], got[:, 0::2], got[:, 1::2]
+    margin = 0.02  # (fp32 accumulation against fp64: leave the values this close to the limit out)
+    assert int((gate_w > 7 + margin).sum()) > 50 and int((up_w.abs() > 7 + margin).sum()) > 50
+    assert torch.all(gate_g[gate_w > 7 + margin] > 7)
+    assert torch.all(up_g[up_w.abs() > 7 + margin].abs() > 7)
+    assert torch.all(gate_g[gate_w < 7 - margin] <= 7) and torch.all(up_g[up_w.abs() < 7 - margin].abs() <= 7)
+    inside = want.abs() < 6.9
+    assert float((got[inside] - want[inside]).abs().max()) < 0.04  # (within a rounding step of the fp64 value)

@@ -108,6 +108,21 @@ __device__ inline void glu_backward(float G, float U, float dh, float &dG, float
   dG = (G > kGluLimit) ? 0.0f : dgl * (s + g * s * (1.0f - s) * kGluAlpha);
 }
 
+// A pre-activation as the backward will read it back: rounded to T, except that a value beyond the clamp limit whose
+// rounding lands on the limit itself is stored one step further out.  glu_backward tests the stored value against the
+// limit; without this, the values in (7, 7.016] of a bf16 run would pass a gradient that the fp32 value, and the
+// forward, clamp away (a few elements in ten thousand, but each one wrong by its whole size).  `up`: the up half is
+// clamped on both sides, the gate half from above only.
+template <typename T> __device__ inline T pre_activation_store(float v, bool up) {
+  T r = ElemTraits<T>::from_f32(v);
+  if constexpr (sizeof(T) == 2) {
+    const uint16_t lim = __builtin_bit_cast(uint16_t, ElemTraits<T>::from_f32(kGluLimit));  // (exactly representable)
+    uint16_t bits = __builtin_bit_cast(uint16_t, r);
+    if ((bits & 0x7fffu) == lim && (v > kGluLimit || (up && v < -kGluLimit))) r = __builtin_bit_cast(T, (uint16_t)(bits + 1));
+  }
+  return r;
+}
+
 // 16 bytes per lane from global memory straight into LDS at lds_base + lane * 16.
 __device__ inline void copy16_to_lds(const void *uniform_base, uint32_t lane_byte_off, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"

@@ -415,8 +415,8 @@ __device__ inline void run_tile(const GemmArgs &args, const TileInfo &ti, LA &la
             float G = acc[mi][np][v] + bg, U = acc[mi][np + 2][v] + bu;
             C[orow * args.ldc + pair] = ElemTraits<T>::from_f32(glu_forward(G, U));
             if (P != nullptr) {
-              P[orow * args.Nd + 2 * pair] = ElemTraits<T>::from_f32(G);
-              P[orow * args.Nd + 2 * pair + 1] = ElemTraits<T>::from_f32(U);
+              P[orow * args.Nd + 2 * pair] = pre_activation_store<T>(G, false);
+              P[orow * args.Nd + 2 * pair + 1] = pre_activation_store<T>(U, true);
             }
           }
         }

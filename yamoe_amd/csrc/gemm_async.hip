@@ -425,8 +425,9 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
       for (int i = 0; i < 4; ++i) b[4 * q + i] = t[i];
     }
   };
-  // natural column order: value = acc + bias[column]   (the plain product, or the pre-activations)
-  auto stage_biased = [&]() {
+  // natural column order: value = acc + bias[column]   (the plain product, or, with `pre`, the pre-activations as the
+  // backward reads them: even columns gate, odd columns up)
+  auto stage_biased = [&](auto pre) {
     constexpr int stride = kBN * 2 + 16;
     char *lp = lds + (wm * 32 + rl) * stride + (wn * 32 + 4 * g) * 2;  // one address per lane, the rest are constants
 #pragma unroll
@@ -438,8 +439,16 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const f32x16 &a = acc[mi][ni];
-          u32x2 v = {pack2<T>(a[4 * q] + b[4 * q], a[4 * q + 1] + b[4 * q + 1]),
-                     pack2<T>(a[4 * q + 2] + b[4 * q + 2], a[4 * q + 3] + b[4 * q + 3])};
+          u32x2 v;
+          if constexpr (decltype(pre)::value) {
+            typedef T T2 __attribute__((ext_vector_type(2)));
+            T2 lo = {pre_activation_store<T>(a[4 * q] + b[4 * q], false), pre_activation_store<T>(a[4 * q + 1] + b[4 * q + 1], true)};
+            T2 hi = {pre_activation_store<T>(a[4 * q + 2] + b[4 * q + 2], false), pre_activation_store<T>(a[4 * q + 3] + b[4 * q + 3], true)};
+            v = (u32x2){__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi)};
+          } else {
+            v = (u32x2){pack2<T>(a[4 * q] + b[4 * q], a[4 * q + 1] + b[4 * q + 1]),
+                        pack2<T>(a[4 * q + 2] + b[4 * q + 2], a[4 * q + 3] + b[4 * q + 3])};
+          }
           *(u32x2 *)(lp + mi * 64 * stride + (ni * 64 + 8 * q) * 2) = v;
         }
     }
@@ -495,12 +504,12 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
     }
   }
   if constexpr (EPI == EPI_STORE) {
-    stage_biased();
+    stage_biased(std::false_type());
     __syncthreads();
     store_rows((T *)args.C, args.ldc, n0, kBN, args.Nd);
   } else {
     if (args.C2 != nullptr) {  // pre-activations for the backward: the biased product itself
-      stage_biased();
+      stage_biased(std::true_type());
       __syncthreads();
       store_rows((T *)args.C2, args.Nd, n0, kBN, args.Nd);
       __syncthreads();

@@ -180,8 +180,8 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == kStreamWaves ? 2 : 1) void str
       ((T *)args.C)[orow * args.ldc + (col >> 1)] = ElemTraits<T>::from_f32(glu_forward(x0, x1));
       if (args.C2 != nullptr) {
         T *P = (T *)args.C2 + orow * args.Nd + col;
-        P[0] = ElemTraits<T>::from_f32(x0);
-        P[1] = ElemTraits<T>::from_f32(x1);
+        P[0] = pre_activation_store<T>(x0, false);
+        P[1] = pre_activation_store<T>(x1, true);
       }
     } else {
       T *O = (T *)args.C + orow * args.ldc + col;
