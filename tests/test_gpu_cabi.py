@@ -1,6 +1,6 @@
 """The whole-op entry points of the C ABI driven the way another host would drive them: through ctypes only, with
-caller-owned outputs and one caller-owned workspace that is reused from call to call (the sequence INTEGRATION.md
-shows for a host that replaces torch-ext/torch_binding.cpp:58-83).  Results against the oracle."""
+caller-owned outputs and one caller-owned workspace that is reused from call to call (the sequence a host follows
+that replaces torch-ext/torch_binding.cpp:58-83: workspace query, forward, backward).  Results against the oracle."""
 import ctypes
 
 import pytest
