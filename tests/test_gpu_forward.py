@@ -223,3 +223,32 @@ def test_forward_and_backward_replay_in_a_hip_graph(gpu):
             assert torch.equal(got, want), rep
         yamoe_amd.experts(*a, T, E, K)                        # eager work between replays
         torch.cuda.synchronize()
+
+
+def test_two_streams_at_once(gpu):
+    """Calls on different streams share nothing but read-only per-device flags (each call carves its own workspace):
+    two problems of different shapes and dtypes, forward and backward, issued alternately on two streams without a
+    synchronisation in between, give the results of the same calls made one after the other, bit for bit."""
+    import yamoe_amd
+    shapes = [(900, 256, 128, 8, 2, torch.bfloat16, 5), (300, 192, 320, 4, 3, torch.float16, 6)]
+    work, serial = [], []
+    for T, H, I, E, K, dtype, seed in shapes:
+        d = make_inputs(T, H, I, E, K, dtype, seed=seed, w_std=0.05, bias_std=0.1, zipf=0.5)
+        g = to_dev(d, gpu)
+        gy = torch.randn(T, H, generator=torch.Generator().manual_seed(seed)).to(dtype).to(gpu)
+        work.append((gy, args(g), T, E, K))
+    for gy, a, T, E, K in work:
+        serial.append([yamoe_amd.experts(*a, T, E, K)] + list(yamoe_amd.experts_backward(gy, *a, T, E, K)))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for rep in range(3):
+        got = [[], []]
+        for it in range(4):  # alternate, so that launches of the two problems interleave on the device
+            for i, (gy, a, T, E, K) in enumerate(work):
+                with torch.cuda.stream(streams[i]):
+                    r = [yamoe_amd.experts(*a, T, E, K)] + list(yamoe_amd.experts_backward(gy, *a, T, E, K))
+                got[i] = r
+        torch.cuda.synchronize()
+        for i in range(2):
+            for x, y in zip(got[i], serial[i]):
+                assert torch.equal(x, y), (rep, i)
