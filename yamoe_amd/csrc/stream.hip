@@ -7,13 +7,13 @@
 // loads (a wave reads 32 rows x 256 contiguous bytes), transposes it in registers and feeds it to
 // eight v_mfma_f32_16x16x32 instructions whose 16-row A operand is the expert's (zero-padded)
 // activations.  No LDS is touched until the final cross-wave reduction.  Two steps of loads are
-// kept in flight per wave, 8 waves per CU.
+// kept in flight per wave, at least 8 waves per CU.
 //
 // A launch that can hold only a few experts (a handful of tokens: at most kStreamFewBlocks workgroups) has too few
 // workgroups to keep HBM busy that way: 4 experts x 23 slabs with two steps of 8 KB in flight per wave are 6 MB on
 // the way, where 8 TB/s x 2 us of latency want 16 MB.  Such a launch takes 8 waves per workgroup with three steps in
-// flight each instead (a workgroup per CU; 16 waves would leave a wave 128 registers, not enough for two steps), folded
-// into the first four before the same finish.
+// flight each instead (a workgroup per CU; 16 waves with two steps each measured 3 % slower), folded into the first
+// four before the same finish.
 //
 // The lane that holds accumulator column c of MFMA j owns output column 8c + j, so the 8
 // accumulators of a lane are 8 consecutive output columns: the interleaved (gate, up) pairs of the
