@@ -97,7 +97,8 @@ def test_padded_gather_bit_exact(gpu, dtype, T, H, E, C, K):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.float64])
 @pytest.mark.parametrize("T,H,E,C,K,weighted", [(64, 128, 8, 4, 2, True), (300, 2880, 32, 50, 4, True),
-                                                (17, 36, 3, 40, 1, False), (90, 130, 4, 1000, 3, True)])
+                                                (17, 36, 3, 40, 1, False), (90, 130, 4, 1000, 3, True),
+                                                (5, 128, 32, 0, 2, True)])   # capacity 0: an empty src, y untouched
 def test_padded_scatter(gpu, dtype, T, H, E, C, K, weighted):
     import yamoe_amd
     print("scatter %s T=%d H=%d E=%d C=%d K=%d" % (dtype, T, H, E, C, K), flush=True)

@@ -337,7 +337,7 @@ extern "C" int yamoe_padded_scatter(const void *src, const int32_t *indices, con
                                     void *workspace, size_t workspace_bytes, void *stream) {
   if (T_ < 0 || H <= 0 || E <= 0 || C < 0 || top_k <= 0) { set_error("yamoe_padded_scatter: bad size"); return YAMOE_E_ARG; }
   const int S = T_ * top_k;
-  if (S == 0) return 0;
+  if (S == 0 || C == 0) return 0;  // (a capacity of zero keeps no row: y stays as it is, and src may be an empty tensor)
   if (!src || !indices || !bins || !y || !workspace || workspace_bytes < yamoe_padded_scatter_workspace_bytes(S)) {
     set_error("yamoe_padded_scatter: null pointer or workspace too small");
     return YAMOE_E_ARG;
