@@ -9,6 +9,9 @@
 
 namespace yamoe {
 
+#ifndef YAMOE_COMBINE_SPLIT_T
+#define YAMOE_COMBINE_SPLIT_T 1024
+#endif
 constexpr int kRowThreads = 256;
 constexpr int kRowWaves = kRowThreads / kWave;
 
@@ -49,20 +52,22 @@ __device__ inline float slot_weight(const T *rw, const void *idx, int t, int k, 
 }
 
 // out[t,:] = sum_k w(t,k) * y_perm[inv_pos[t*K+k],:]
-// One wave per token.  The K (position, weight) pairs of the token are fetched once (up to kMaxSlots of
-// them sit in registers), then every lane streams its 16-byte chunks of the K rows.
+// `split` waves per token (1, or the 4 of a workgroup when there are few tokens: a lone wave goes through a 2880-wide
+// row in six dependent rounds of loads).  The K (position, weight) pairs of the token are fetched once (up to
+// kMaxSlots of them sit in registers), then every lane streams its 16-byte chunks of the K rows.
 constexpr int kMaxSlots = 8;
 
 template <typename T, bool I64>
 __global__ __launch_bounds__(kRowThreads) void combine_kernel(
     const T *__restrict__ y_perm, const int *__restrict__ inv_pos, const void *__restrict__ idx,
-    const T *__restrict__ rw, int rw_cols, T *__restrict__ out, int Tn, int K, int E, int H) {
+    const T *__restrict__ rw, int rw_cols, T *__restrict__ out, int Tn, int K, int E, int H, int split) {
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = blockIdx.x * kRowWaves + threadIdx.x / kWave;
   const int n_waves = gridDim.x * kRowWaves;
   constexpr int V = ElemTraits<T>::kVec;
   const bool vec_ok = (H % V) == 0;
-  for (int t = wave; t < Tn; t += n_waves) {
+  const int part = wave % split, stride = kWave * split;
+  for (int t = wave / split; t < Tn; t += n_waves / split) {
     T *dst = out + (size_t)t * H;
     if (vec_ok && K <= kMaxSlots) {
       int pos[kMaxSlots];
@@ -76,7 +81,7 @@ __global__ __launch_bounds__(kRowThreads) void combine_kernel(
           if (pos[k] >= 0) w[k] = slot_weight<T, I64>(rw, idx, t, k, K, E, rw_cols);
         }
       }
-      for (int c = lane; c < H / V; c += kWave) {
+      for (int c = part * kWave + lane; c < H / V; c += stride) {
         float acc[V];
 #pragma unroll
         for (int j = 0; j < V; ++j) acc[j] = 0.0f;
@@ -95,7 +100,7 @@ __global__ __launch_bounds__(kRowThreads) void combine_kernel(
         ((u32x4 *)dst)[c] = o;
       }
     } else {
-      for (int c = lane; c < H; c += kWave) {
+      for (int c = part * kWave + lane; c < H; c += stride) {
         float acc = 0.0f;
         for (int k = 0; k < K; ++k) {
           int pos = inv_pos[(size_t)t * K + k];
@@ -354,13 +359,14 @@ int launch_combine(const void *y_perm, const int *inv_pos, const void *idx, int 
                    const void *rw, int rw_cols, void *out, int Tn, int K, int E, int H,
                    hipStream_t stream) {
   if (Tn == 0) return 0;
-  int blocks = min(ceil_div(Tn, kRowWaves), 256 * 16);
+  const int split = Tn <= YAMOE_COMBINE_SPLIT_T ? kRowWaves : 1;  // (the grid is a whole number of groups of `split` waves)
+  int blocks = min(ceil_div(Tn * split, kRowWaves), 256 * 16);
   if (idx_i64)
     hipLaunchKernelGGL((combine_kernel<T, true>), dim3(blocks), dim3(kRowThreads), 0, stream,
-                       (const T *)y_perm, inv_pos, idx, (const T *)rw, rw_cols, (T *)out, Tn, K, E, H);
+                       (const T *)y_perm, inv_pos, idx, (const T *)rw, rw_cols, (T *)out, Tn, K, E, H, split);
   else
     hipLaunchKernelGGL((combine_kernel<T, false>), dim3(blocks), dim3(kRowThreads), 0, stream,
-                       (const T *)y_perm, inv_pos, idx, (const T *)rw, rw_cols, (T *)out, Tn, K, E, H);
+                       (const T *)y_perm, inv_pos, idx, (const T *)rw, rw_cols, (T *)out, Tn, K, E, H, split);
   return check_launch("combine_kernel");
 }
 
