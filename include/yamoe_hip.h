@@ -99,8 +99,10 @@ int yamoe_combine(const void *y_perm, const int32_t *inv_pos, const void *router
  *   down:    y_perm[p,:] = act[p,:] . Wd[e] + bd[e]
  * Rows p with rank >= capacity inside their expert are not computed.
  * `schedule` is the workspace region filled by yamoe_build_schedule: experts with
- * 1..stream_max_rows kept rows (at most 16; 16-bit dtypes only, pass 0 for fp32) are
+ * 1..stream_max_rows kept rows (at most 32; 16-bit dtypes only, pass 0 for fp32) are
  * listed for the weight-streaming kernel, the others are cut into 256-row MFMA tiles.
+ * A limit above 16 applies only when no expert has more kept rows than the limit;
+ * otherwise experts with up to 16 rows stream and the others are tiled.
  * yamoe_gate_up / yamoe_down launch both kernels; each walks its own list. */
 size_t yamoe_schedule_bytes(int32_t N, int32_t E);
 int yamoe_build_schedule(const int32_t *counts, const int32_t *offsets, int32_t N, int32_t E,

@@ -102,11 +102,15 @@ def test_permute_and_combine(gpu, dtype, T, K, E, H):
 
 
 @pytest.mark.parametrize("N,E,C,stream_rows", [(256, 128, 64, 16), (16384, 32, 4096, 16), (65536, 128, 300, 16),
-                                               (1000, 700, 5, 0), (40, 3, 40, 16)])
+                                               (1000, 700, 5, 0), (40, 3, 40, 16),
+                                               (300, 40, 30, 32),      # every expert within 32 rows: all of them stream
+                                               (300, 40, 300, 32),     # some beyond 32: the limit falls back to 16
+                                               (2000, 64, 32, 32)])    # capacity 32 keeps everybody within the limit
 def test_schedule_lists(gpu, N, E, C, stream_rows):
     """The device-built work lists: experts with 1..stream_rows kept rows in the streaming list, the
     rest cut into equal row tiles (as few as 256 rows allow, each a multiple of 32 rows but the last), both in
-    expert order, none dropped, none duplicated."""
+    expert order, none dropped, none duplicated.  A limit above 16 holds only if no expert exceeds it; with such
+    experts present the limit is 16."""
     from yamoe_amd import _cabi
     rng = np.random.default_rng(N * 7 + E)
     p = rng.random(E) ** 4
@@ -116,6 +120,8 @@ def test_schedule_lists(gpu, N, E, C, stream_rows):
     offsets = torch.from_numpy(r["offsets"]).to(gpu)
     sched = _cabi.build_schedule(counts, offsets, N, C, stream_rows).cpu().numpy()
     want_tiles, want_small = [], []
+    if stream_rows > 16 and int(np.minimum(r["counts"], C).max()) > stream_rows:
+        stream_rows = 16
     for e in range(E):
         kept = min(int(r["counts"][e]), C)
         if kept == 0:

@@ -16,8 +16,10 @@ constexpr int kWave = 64;
 constexpr float kGluLimit = 7.0f;
 constexpr float kGluAlpha = 1.702f;
 
-// Experts with at most this many kept rows take the weight-streaming path.
-constexpr int kStreamMaxRows = 16;
+// Experts with at most this many kept rows take the weight-streaming path: 32 when that covers every expert of the
+// call, 16 when some experts need the tile kernels anyway.
+constexpr int kStreamMaxRows = 32;
+constexpr int kStreamMixedRows = 16;
 
 typedef __bf16 bf16_t;
 typedef _Float16 f16_t;
@@ -177,6 +179,8 @@ __host__ __device__ inline int sched_max_row_tiles(int N, int E) {
 // Upper bound of the row-tile count when experts with at most `small_rows` kept rows are not tiled (they are on
 // the streaming list): only N / (small_rows + 1) experts can hold more rows than that.  Used for grid sizes only.
 __host__ __device__ inline int sched_grid_row_tiles(int N, int E, int small_rows) {
+  // (the list may have been built with the lower of the two streaming limits)
+  if (small_rows > kStreamMixedRows) small_rows = kStreamMixedRows;
   int tiled = N / (small_rows + 1);
   if (tiled > E) tiled = E;
   return N / kRowTile + tiled + 1;

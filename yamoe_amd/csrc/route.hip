@@ -148,6 +148,19 @@ __device__ inline void build_schedule_wave(const int *counts, const int *offsets
   int *row_tiles = sched + kSchedHeader;
   int *small = row_tiles + 8 * sched_max_row_tiles(N, E);
   int n_tiles = 0, n_small = 0, n_active = 0, n_kept = 0;
+  // Experts of 17 to 32 rows stream only when every expert streams: next to experts that need the tile kernels anyway
+  // they are better off as tiles (two half-filled launches one after the other are slower than one: 0.35 against
+  // 0.31 ms for 32 experts of about 32 rows, where 0.27 against 0.31 ms is gained when all of them have at most 32).
+  if (stream_max_rows > kStreamMixedRows) {
+    int most = 0;
+    for (int base = 0; base < E; base += kWave) {
+      int e = base + lane;
+      int kept = e < E ? min(counts[e], capacity) : 0;
+      most = max(most, kept);
+    }
+    for (int d = kWave / 2; d > 0; d >>= 1) most = max(most, __shfl_xor(most, d));
+    if (most > stream_max_rows) stream_max_rows = kStreamMixedRows;
+  }
   for (int base = 0; base < E; base += kWave) {
     int e = base + lane;
     int kept = e < E ? min(counts[e], capacity) : 0;

@@ -1,4 +1,4 @@
-// Weight-streaming path for experts with at most 16 kept rows (the decode regime).
+// Weight-streaming path for experts with at most 32 kept rows (the decode regime).
 //
 // Such an expert does 2*rows flops per weight element, far below the machine balance, so the job
 // is to pull each expert's weights through the chip once at HBM rate.  A workgroup owns one
@@ -6,7 +6,7 @@
 // of the slab round-robin; in a step every lane fetches an 8(k) x 8(column) block as eight 16-byte
 // loads (a wave reads 32 rows x 256 contiguous bytes), transposes it in registers and feeds it to
 // eight v_mfma_f32_16x16x32 instructions whose 16-row A operand is the expert's (zero-padded)
-// activations.  No LDS is touched until the final cross-wave reduction.  Two steps of loads are
+// activations (an expert with 17 to 32 rows has two such operands and runs every column operand through both).  No LDS is touched until the final cross-wave reduction.  Two steps of loads are
 // kept in flight per wave, at least 8 waves per CU.
 //
 // A launch that can hold only a few experts (a handful of tokens: at most kStreamFewBlocks workgroups) has too few
@@ -54,40 +54,45 @@ struct StreamArgs {
   int a_div, Kd, Nd, lda, ldc, n_slabs, N, E;
 };
 
-template <typename T, bool GLU, bool GATHER, int WAVES, int DEPTH>
-__global__ __launch_bounds__(64 * WAVES, WAVES == kStreamWaves ? 2 : 1) void stream_gemm_kernel(const StreamArgs args) {
-  __shared__ float red[kStreamWaves * 8 * 4 * kWave];  // [wave][j][v][lane]
+// One (expert, slab) of RB blocks of 16 rows (RB = 1: up to 16 rows, RB = 2: 17 to 32): the weights are fetched once
+// and every column operand built from them goes through RB MFMAs.
+template <typename T, bool GLU, bool GATHER, int WAVES, int DEPTH, int RB>
+__device__ inline void stream_slab(const StreamArgs &args, float *red, const int expert, const int first, const int rows,
+                                   const int slab) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const ScheduleView sv = schedule_view(args.sched, args.N, args.E);
-  const int n_small = sv.hdr[1];
-  const int s = blockIdx.x / args.n_slabs;
-  if (s >= n_small) return;
-  const int slab = blockIdx.x - s * args.n_slabs;
-  const int expert = sv.small[4 * s], first = sv.small[4 * s + 1], rows = sv.small[4 * s + 2];
-
   const int c16 = lane & 15, g = lane >> 4;
   const int col0 = slab * kSlabCols + c16 * 8;  // first of this lane's 8 output columns
   const bool col_ok = col0 < args.Nd;
   const T *Bp = (const T *)args.B + (long long)expert * args.Kd * args.Nd + col0;
 
-  // A operand: row c16 of the expert (zero beyond `rows`), 8 consecutive k starting at 8 g
-  const bool a_ok = c16 < rows;
-  long long a_src = first + (a_ok ? c16 : 0);
-  if (GATHER) a_src = args.a_rows[a_src] / args.a_div;
-  const T *Ap = (const T *)args.A + a_src * args.lda + g * 8;
-
-  f32x4v acc[8];
+  // A operand of block b: row 16 b + c16 of the expert (zero beyond `rows`), 8 consecutive k starting at 8 g
+  bool a_ok[RB];
+  const T *Ap[RB];
 #pragma unroll
-  for (int j = 0; j < 8; ++j) acc[j] = (f32x4v){0.f, 0.f, 0.f, 0.f};
+  for (int b = 0; b < RB; ++b) {
+    a_ok[b] = 16 * b + c16 < rows;
+    long long a_src = first + (a_ok[b] ? 16 * b + c16 : 0);
+    if (GATHER) a_src = args.a_rows[a_src] / args.a_div;
+    Ap[b] = (const T *)args.A + a_src * args.lda + g * 8;
+  }
+
+  f32x4v acc[RB][8];
+#pragma unroll
+  for (int b = 0; b < RB; ++b)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[b][j] = (f32x4v){0.f, 0.f, 0.f, 0.f};
 
   const int n_steps = (args.Kd + 31) / 32;
-  u32x4 bw[DEPTH][8], aw[DEPTH];
+  u32x4 bw[DEPTH][8], aw[DEPTH][RB];
 
-  auto fetch = [&](int step, u32x4 (&bw)[8], u32x4 &aw) {
+  auto fetch = [&](int step, u32x4 (&bw)[8], u32x4 (&aw)[RB]) {
     int k0 = step * 32;
     int ka = k0 + g * 8;
-    aw = (u32x4){0, 0, 0, 0};
-    if (a_ok && ka < args.Kd) aw = *(const u32x4 *)(Ap + k0);
+#pragma unroll
+    for (int b = 0; b < RB; ++b) {
+      aw[b] = (u32x4){0, 0, 0, 0};
+      if (a_ok[b] && ka < args.Kd) aw[b] = *(const u32x4 *)(Ap[b] + k0);
+    }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       int k = ka + i;
@@ -96,14 +101,15 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == kStreamWaves ? 2 : 1) void str
       bw[i] = v;
     }
   };
-  auto consume = [&](const u32x4 (&bw)[8], const u32x4 &aw) {
+  auto consume = [&](const u32x4 (&bw)[8], const u32x4 (&aw)[RB]) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
       u32x4 col;
 #pragma unroll
       for (int d = 0; d < 4; ++d) col[d] = __builtin_amdgcn_perm(bw[2 * d + 1][j >> 1], bw[2 * d][j >> 1], sel);
-      acc[j] = Mma16<T>::run(aw, col, acc[j]);
+#pragma unroll
+      for (int b = 0; b < RB; ++b) acc[b][j] = Mma16<T>::run(aw[b], col, acc[b][j]);
     }
   };
 
@@ -124,71 +130,86 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == kStreamWaves ? 2 : 1) void str
     }
   }
 
-  // ---- reduce the partial sums and finish ---------------------------------------------------------
-  // more than four waves: waves 4r .. 4r+3 hand their sums to waves 0 .. 3, one group after the other (a fixed order)
-  for (int r = 1; r < WAVES / kStreamWaves; ++r) {
-    if (wave / kStreamWaves == r) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) red[(((wave - kStreamWaves * r) * 8 + j) * 4 + v) * kWave + lane] = acc[j][v];
-    }
-    __syncthreads();
-    if (wave < kStreamWaves) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) acc[j][v] += red[((wave * 8 + j) * 4 + v) * kWave + lane];
-    }
-    __syncthreads();
-  }
-  if (wave < kStreamWaves) {
-#pragma unroll
-    for (int j = 0; j < 8; ++j)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) red[((wave * 8 + j) * 4 + v) * kWave + lane] = acc[j][v];
-  }
-  __syncthreads();
-  if (wave >= kStreamWaves) return;  // (after the last workgroup barrier)
-
-  // wave w finishes accumulator columns j = 2w, 2w+1 (one gate/up pair per lane)
-  float sum[2][4];
-#pragma unroll
-  for (int jj = 0; jj < 2; ++jj)
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      float t = 0.f;
-#pragma unroll
-      for (int w = 0; w < kStreamWaves; ++w) t += red[((w * 8 + 2 * wave + jj) * 4 + v) * kWave + lane];
-      sum[jj][v] = t;
-    }
-  const int col = col0 + 2 * wave;
-  if (!col_ok) return;
+  // ---- reduce the partial sums and finish, one block of 16 rows after the other -------------------------------
+  const int col = col0 + 2 * wave;  // wave w (of the first four) finishes accumulator columns j = 2w, 2w+1: one (gate, up) pair per lane
   float b0 = 0.f, b1 = 0.f;
-  if (args.bias != nullptr) {
+  if (wave < kStreamWaves && col_ok && args.bias != nullptr) {
     const T *bp = (const T *)args.bias + (long long)expert * args.Nd + col;
     b0 = ElemTraits<T>::to_f32(bp[0]);
     b1 = ElemTraits<T>::to_f32(bp[1]);
   }
 #pragma unroll
-  for (int v = 0; v < 4; ++v) {
-    int r = g * 4 + v;
-    if (r >= rows) continue;
-    long long orow = first + r;
-    float x0 = sum[0][v] + b0, x1 = sum[1][v] + b1;
-    if (GLU) {
-      ((T *)args.C)[orow * args.ldc + (col >> 1)] = ElemTraits<T>::from_f32(glu_forward(x0, x1));
-      if (args.C2 != nullptr) {
-        T *P = (T *)args.C2 + orow * args.Nd + col;
-        P[0] = pre_activation_store<T>(x0, false);
-        P[1] = pre_activation_store<T>(x1, true);
+  for (int b = 0; b < RB; ++b) {
+    // more than four waves: waves 4r .. 4r+3 hand their sums to waves 0 .. 3, one group after the other (a fixed order)
+    for (int r = 1; r < WAVES / kStreamWaves; ++r) {
+      if (wave / kStreamWaves == r) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) red[(((wave - kStreamWaves * r) * 8 + j) * 4 + v) * kWave + lane] = acc[b][j][v];
       }
-    } else {
-      T *O = (T *)args.C + orow * args.ldc + col;
-      O[0] = ElemTraits<T>::from_f32(x0);
-      O[1] = ElemTraits<T>::from_f32(x1);
+      __syncthreads();
+      if (wave < kStreamWaves) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) acc[b][j][v] += red[((wave * 8 + j) * 4 + v) * kWave + lane];
+      }
+      __syncthreads();
     }
+    if (wave < kStreamWaves) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[((wave * 8 + j) * 4 + v) * kWave + lane] = acc[b][j][v];
+    }
+    __syncthreads();
+    if (wave < kStreamWaves && col_ok) {
+      float sum[2][4];
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          float t = 0.f;
+#pragma unroll
+          for (int w = 0; w < kStreamWaves; ++w) t += red[((w * 8 + 2 * wave + jj) * 4 + v) * kWave + lane];
+          sum[jj][v] = t;
+        }
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        int r = 16 * b + g * 4 + v;
+        if (r >= rows) continue;
+        long long orow = first + r;
+        float x0 = sum[0][v] + b0, x1 = sum[1][v] + b1;
+        if (GLU) {
+          ((T *)args.C)[orow * args.ldc + (col >> 1)] = ElemTraits<T>::from_f32(glu_forward(x0, x1));
+          if (args.C2 != nullptr) {
+            T *P = (T *)args.C2 + orow * args.Nd + col;
+            P[0] = pre_activation_store<T>(x0, false);
+            P[1] = pre_activation_store<T>(x1, true);
+          }
+        } else {
+          T *O = (T *)args.C + orow * args.ldc + col;
+          O[0] = ElemTraits<T>::from_f32(x0);
+          O[1] = ElemTraits<T>::from_f32(x1);
+        }
+      }
+    }
+    if (b + 1 < RB) __syncthreads();  // the next block reuses the buffer
   }
+}
+
+template <typename T, bool GLU, bool GATHER, int WAVES, int DEPTH>
+__global__ __launch_bounds__(64 * WAVES, WAVES == kStreamWaves ? 2 : 1) void stream_gemm_kernel(const StreamArgs args) {
+  __shared__ float red[kStreamWaves * 8 * 4 * kWave];  // [wave][j][v][lane]
+  const ScheduleView sv = schedule_view(args.sched, args.N, args.E);
+  const int n_small = sv.hdr[1];
+  const int s = blockIdx.x / args.n_slabs;
+  if (s >= n_small) return;
+  const int slab = blockIdx.x - s * args.n_slabs;
+  const int expert = sv.small[4 * s], first = sv.small[4 * s + 1], rows = sv.small[4 * s + 2];
+  if (rows > 16) stream_slab<T, GLU, GATHER, WAVES, DEPTH, 2>(args, red, expert, first, rows, slab);
+  else stream_slab<T, GLU, GATHER, WAVES, DEPTH, 1>(args, red, expert, first, rows, slab);
 }
 
 template <typename T, bool GLU, bool GATHER>
