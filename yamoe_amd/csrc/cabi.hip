@@ -86,7 +86,8 @@ template <typename T>
 int gemm_async_dgrad(const void *, const int *, int, const void *, void *, const void *, int, int, int, int,
                      const void *, float *, hipStream_t);
 template <typename T>
-int gemm_async_wgrad(const void *, const void *, void *, const int *, const int *, int, int, int, int, hipStream_t);
+int gemm_async_wgrad(const void *, const int *, int, int, const void *, void *, const int *, const int *, int, int, int,
+                     int, hipStream_t);
 bool gemm_async_supported(int Kd, int Nd, int lda, int ldb, long long a_span_bytes);
 bool gemm_f32_supported(int Kd, int Nd, int lda, int ldb, long long a_span_bytes);
 int gemm_f32_gate_up(const void *, const int *, const void *, const void *, void *, void *, const void *, int, int, int,
@@ -139,12 +140,23 @@ static int tiles_dgrad(const void *g, const int *g_rows, int g_div, long long g_
   return gemm_dgrad<T>(g, g_rows, g_div, w, out, sched, N, E, Kd, Nd, dot_with, dot_part, stream);
 }
 
+// True when the weight-gradient kernel for this dtype and shape can gather the rows of its left operand by token
+// (the register-staged kernel wants them in expert order).
+template <typename T> static bool wgrad_gathers(int Md, int Nd) {
+  if constexpr (sizeof(T) == 2) return wgrad_async_supported(Md, Nd);
+  return false;
+}
+
+// l_rows (with wgrad_gathers only): sorted row p of the left operand is row l_rows[p] / l_div of L; the list holds
+// n_rows values below n_rows and is followed by at least 32 readable ints
 template <typename T>
-static int tiles_wgrad(const void *L, const void *R, void *dW, const int *counts, const int *offsets, int capacity, int E,
-                       int Md, int Nd, hipStream_t stream) {
+static int tiles_wgrad(const void *L, const int *l_rows, int l_div, int n_rows, const void *R, void *dW,
+                       const int *counts, const int *offsets, int capacity, int E, int Md, int Nd, hipStream_t stream) {
   if constexpr (sizeof(T) == 2) {
-    if (wgrad_async_supported(Md, Nd)) return gemm_async_wgrad<T>(L, R, dW, counts, offsets, capacity, E, Md, Nd, stream);
+    if (wgrad_async_supported(Md, Nd))
+      return gemm_async_wgrad<T>(L, l_rows, l_div, n_rows, R, dW, counts, offsets, capacity, E, Md, Nd, stream);
   }
+  if (l_rows != nullptr) { set_error("tiles_wgrad: this kernel takes its rows in expert order"); return YAMOE_E_ARG; }
   return gemm_wgrad<T>(L, R, dW, counts, offsets, capacity, E, Md, Nd, stream);
 }
 
@@ -240,7 +252,9 @@ static size_t carve_backward(const yamoe_problem *p, void *ws, BackwardBuffers *
   size_t used = carve_forward(p, ws, &b->f);
   const size_t N = (size_t)p->T * p->K, es = dtype_size(p->dtype);
   Carver c(ws ? (char *)ws + used : nullptr);
-  b->x_perm = c.take(N * p->H * es);
+  // hidden rows in expert order: only where the gate_up weight-gradient kernel cannot gather them itself
+  const bool gathers = es == 2 ? wgrad_gathers<bf16_t>(p->H, 2 * p->I) : wgrad_gathers<float>(p->H, 2 * p->I);
+  b->x_perm = gathers ? nullptr : c.take(N * p->H * es);
   b->pre = c.take(N * 2 * p->I * es);
   b->g_y_perm = c.take(N * p->H * es);
   b->d_pre = c.take(N * 2 * p->I * es);
@@ -313,7 +327,8 @@ static int backward_impl(const yamoe_problem *p, const void *gy, const void *x, 
   YAMOE_TRY(route_and_schedule(idx, p->idx_i64, N, E, cap, b.f.sorted_expert, b.f.sorted_idx, b.f.counts, b.f.offsets,
                                b.f.inv_pos, b.f.route_ws, b.f.route_ws_bytes, 0, b.f.schedule, b.f.schedule_bytes, st));
   // forward recompute of the first product only: activations and pre-activations
-  YAMOE_TRY(launch_permute<T>(x, b.f.sorted_idx, b.x_perm, N, p->K, H, stream));
+  const bool gathers = wgrad_gathers<T>(H, 2 * I);
+  if (!gathers) YAMOE_TRY(launch_permute<T>(x, b.f.sorted_idx, b.x_perm, N, p->K, H, stream));
   YAMOE_TRY(tiles_gate_up<T>(x, b.f.sorted_idx, wgu, bgu, b.f.act, b.pre, b.f.schedule, N, p->K, E, H, I, 0, stream));
   // combine backward: g_y_perm = grad_out[tok] * w, and the bias part of the routing gradient
   YAMOE_TRY(launch_combine_backward<T>(gy, bd, b.f.sorted_idx, b.f.inv_pos, idx, p->idx_i64, rw, p->rw_cols, b.g_y_perm,
@@ -323,7 +338,8 @@ static int backward_impl(const yamoe_problem *p, const void *gy, const void *x, 
   YAMOE_TRY(launch_expert_colsum<T>(b.g_y_perm, b.f.counts, b.f.offsets, cap, d_bd, E, H, stream));
   YAMOE_TRY(tiles_dgrad<T>(gy, b.f.sorted_idx, p->K, (long long)p->T * H * (long long)es, wd, b.d_act, b.f.schedule, N, E,
                            /*Kd=*/H, /*Nd=*/I, b.f.act, b.dot_part, stream));
-  YAMOE_TRY(tiles_wgrad<T>(b.f.act, b.g_y_perm, d_wd, b.f.counts, b.f.offsets, cap, E, /*Md=*/I, /*Nd=*/H, stream));
+  YAMOE_TRY(tiles_wgrad<T>(b.f.act, nullptr, 1, 0, b.g_y_perm, d_wd, b.f.counts, b.f.offsets, cap, E, /*Md=*/I, /*Nd=*/H,
+                           stream));
   // GLU backward (scaled by the routing weight) and the routing gradient
   YAMOE_TRY(glu_backward_rows<T>(b.d_act, b.pre, b.w_sorted, b.dot_part, b.n_part, b.f.sorted_idx, b.f.inv_pos, b.d_pre,
                                  b.row_dot, N, I, stream));
@@ -332,7 +348,14 @@ static int backward_impl(const yamoe_problem *p, const void *gy, const void *x, 
   YAMOE_TRY(launch_expert_colsum<T>(b.d_pre, b.f.counts, b.f.offsets, cap, d_bgu, E, 2 * I, stream));
   YAMOE_TRY(tiles_dgrad<T>(b.d_pre, nullptr, 1, 0, wgu, b.d_x_perm, b.f.schedule, N, E, /*Kd=*/2 * I, /*Nd=*/H, nullptr,
                            nullptr, stream));
-  YAMOE_TRY(tiles_wgrad<T>(b.x_perm, b.d_pre, d_wgu, b.f.counts, b.f.offsets, cap, E, /*Md=*/H, /*Nd=*/2 * I, stream));
+  // (the hidden rows gathered by token where the kernel can do that; check_problem keeps hidden below 4 GiB, and
+  // sorted_idx is followed in the workspace by inv_pos and the rest: readable well past its end)
+  if (gathers)
+    YAMOE_TRY(tiles_wgrad<T>(x, b.f.sorted_idx, p->K, N, b.d_pre, d_wgu, b.f.counts, b.f.offsets, cap, E, /*Md=*/H,
+                             /*Nd=*/2 * I, stream));
+  else
+    YAMOE_TRY(tiles_wgrad<T>(b.x_perm, nullptr, 1, 0, b.d_pre, d_wgu, b.f.counts, b.f.offsets, cap, E, /*Md=*/H, /*Nd=*/2 * I,
+                             stream));
   // permute backward: d_hidden[t] = sum_k d_x_perm[inv_pos[t,k]]
   YAMOE_TRY(launch_combine<T>(b.d_x_perm, b.f.inv_pos, idx, p->idx_i64, nullptr, p->K, d_x, p->T, p->K, E, H, stream));
   return 0;

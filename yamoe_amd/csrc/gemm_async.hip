@@ -679,10 +679,13 @@ static int launch(const Args &args, int max_row_tiles, hipStream_t stream) {
 // whatever follows in memory (the caller keeps that readable) and the wave that issued them overwrites them with
 // zeros in LDS before anybody reads the slab.
 struct WgradArgs {
-  const void *A;  // [N, Md] rows in expert order
+  const void *A;  // [N, Md] rows in expert order; with a_rows: [*, Md], sorted row p is row a_rows[p] / a_div of it
   const void *B;  // [N, Nd]
   void *C;        // [E, Md, Nd]
   const int *counts, *offsets;
+  const int *a_rows;
+  FastDiv a_div;
+  int a_rows_max;  // largest value a_rows may hold
   int capacity, E, Md, Nd, n_m_tiles, n_n_tiles;
 };
 
@@ -701,7 +704,7 @@ constexpr int kSmallRing = kSmallStages * (kSmallAStage + kSmallBStage);
 constexpr int kSmallStaging = kSmallBM * (kBN * 2 + 16);
 constexpr int kSmallLds = kSmallRing > kSmallStaging ? kSmallRing : kSmallStaging;
 
-template <typename T, int NMI>
+template <typename T, int NMI, bool GATHER>
 __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid, const int expert, const int m0,
                                             const int n0, const int rows_m, const long long first, const int rows) {
   const int lane = tid & 63;
@@ -731,7 +734,7 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
     int piece = (lane & 15) ^ ((k & 3) << 2);
     int ca = m0 + piece * 8;
     if (ca >= args.Md) ca = m0;
-    a_off[i] = (uint32_t)(k * lda_bytes + (long long)(ca - m0) * (long long)sizeof(T));
+    a_off[i] = (uint32_t)((GATHER ? 0ll : k * lda_bytes) + (long long)(ca - m0) * (long long)sizeof(T));
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -741,18 +744,50 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
     if (cb >= args.Nd) cb = n0;
     b_off[i] = (uint32_t)(k * ldb_bytes + (long long)(cb - n0) * (long long)sizeof(T));
   }
-  const char *a_base = (const char *)((const T *)args.A + first * args.Md + m0);
+  const char *a_base = (const char *)((const T *)args.A + (GATHER ? 0ll : first * args.Md) + m0);
   const char *b_base = (const char *)((const T *)args.B + first * args.Nd + n0);
-  auto copy_a = [&](int slab, int i) {
-    copy16_to_lds(a_base + (long long)slab * kBK * lda_bytes, a_off[i],
+  // Gathered A rows: the four k rows of piece i of a slab are rows a_rows[first + 32*slab + 4*(2*wave + i) + 0..3]
+  // / a_div of A.  The positions are the same for the whole wave, so the look-ups are scalar loads (rows_of), issued
+  // at the start of the half slab whose last slot issues the copy; there the lane picks its row and turns it into a
+  // byte offset (row_bytes).  Positions past the expert's rows (up to 31 past the end of the list: the caller keeps
+  // that readable) hold somebody else's row or anything at all: the value is clamped to the list's range, and what the
+  // copy fetches is zeroed in LDS before use.  The list is read through the constant address space, which makes the loads scalar whatever the
+  // compiler can prove about the memory in between (the list was written by an earlier launch).
+  typedef const __attribute__((address_space(4))) int *ConstInts;
+  ConstInts a_rows = GATHER ? (ConstInts)(uintptr_t)(args.a_rows + first) : (ConstInts)0;
+  auto rows_of = [&](int slab, int i, int (&ix)[4]) {
+    if constexpr (GATHER) {
+      const int k0 = slab * kBK + 4 * (2 * wave + i);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ix[j] = a_rows[k0 + j];
+    }
+  };
+  auto row_bytes = [&](int (&ix)[4]) -> uint32_t {
+    if constexpr (!GATHER) return 0u;
+    // the four values pass through an empty statement: the loads stay where rows_of put them, all four of them, and
+    // what follows is three selects rather than loads under branches
+    int r0 = ix[0], r1 = ix[1], r2 = ix[2], r3 = ix[3];
+    asm volatile("" : "+s"(r0), "+s"(r1), "+s"(r2), "+s"(r3));
+    const bool odd = (lane & 16) != 0, high = (lane & 32) != 0;
+    const int lo = odd ? r1 : r0, hi = odd ? r3 : r2;
+    const uint32_t r = min((uint32_t)(high ? hi : lo), (uint32_t)args.a_rows_max);
+    return (uint32_t)fast_div((int)r, args.a_div) * (uint32_t)lda_bytes;
+  };
+  auto copy_a = [&](int slab, int i, uint32_t row) {
+    copy16_to_lds(a_base + (GATHER ? 0ll : (long long)slab * kBK * lda_bytes), a_off[i] + row,
                   lds0 + (uint32_t)(slab % kSmallStages) * kSmallAStage + (uint32_t)(4 * (2 * wave + i)) * 256u);
+  };
+  auto copy_a_now = [&](int slab, int i) {  // look-up and copy in one go: outside the pipelined loop
+    int ix[4] = {0, 0, 0, 0};
+    rows_of(slab, i, ix);
+    copy_a(slab, i, row_bytes(ix));
   };
   auto copy_b = [&](int slab, int i) {
     copy16_to_lds(b_base + (long long)slab * kBK * ldb_bytes, b_off[i],
                   lds0 + kSmallBRing + (uint32_t)(slab % kSmallStages) * kSmallBStage + (uint32_t)(8 * wave + 2 * i) * 512u);
   };
   auto copy_slab = [&](int slab) {
-    copy_a(slab, 0); copy_b(slab, 0); copy_b(slab, 1); copy_a(slab, 1); copy_b(slab, 2); copy_b(slab, 3);
+    copy_a_now(slab, 0); copy_b(slab, 0); copy_b(slab, 1); copy_a_now(slab, 1); copy_b(slab, 2); copy_b(slab, 3);
   };
   auto zero_tail = [&](int slab) {
 #pragma unroll
@@ -836,10 +871,12 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
     u32x4 v = (u32x4){lo[0], lo[1], hi[0], hi[1]};
     if (is_a) fa[idx] = v; else fb[idx] = v;
   };
-  auto copy_a_c = [&](auto stage, int slab, int i) {
+  auto copy_a_c = [&](auto stage, int slab, int i, uint32_t row) {
     constexpr int ST = decltype(stage)::value;
-    copy16_to_lds(a_base + (long long)slab * kBK * lda_bytes, a_off[i], lds_a_wave + (uint32_t)(ST * kSmallAStage + 4 * i * 256));
+    copy16_to_lds(a_base + (GATHER ? 0ll : (long long)slab * kBK * lda_bytes), a_off[i] + row,
+                  lds_a_wave + (uint32_t)(ST * kSmallAStage + 4 * i * 256));
   };
+
   auto copy_b_c = [&](auto stage, int slab, int i) {
     constexpr int ST = decltype(stage)::value;
     copy16_to_lds(b_base + (long long)slab * kBK * ldb_bytes, b_off[i], lds_b_wave + (uint32_t)(ST * kSmallBStage + 2 * i * 512));
@@ -853,15 +890,20 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
     __builtin_amdgcn_sched_barrier(0);
     {
       constexpr int kC = C::P1 ? 3 : 0, kItems = kC + kFrags;
+      int ix[4] = {0, 0, 0, 0};  // gathered rows: the four rows of the A piece copied in this half slab
 #pragma unroll
       for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
         if (j < kMma) Mma<T>::run(fb0[j & 3], fa0[j >> 2], acc[j >> 2][j & 3]);
         if (j < kSlots) {
 #pragma unroll
           for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
-            if (i < kC) { if (i == 0) copy_a_c(Next2(), s + 2, 1); else copy_b_c(Next2(), s + 2, 1 + i); }
+            if (i < kC) {
+              if (i == 0) { if constexpr (GATHER) rows_of(s + 2, 1, ix); else copy_a_c(Next2(), s + 2, 1, 0u); }
+              else copy_b_c(Next2(), s + 2, 1 + i);
+            }
             else read_frag_c(stage, 1, i - kC, fa1, fb1);
           }
+          if (GATHER && kC > 0 && j == kSlots - 1) copy_a_c(Next2(), s + 2, 1, row_bytes(ix));
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -873,15 +915,20 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
     __builtin_amdgcn_sched_barrier(0);
     {
       constexpr int kC = C::P2 ? 3 : 0, kItems = kC + (C::NEXT ? kFrags : 0);
+      int ix[4] = {0, 0, 0, 0};  // gathered rows: the four rows of the A piece copied in this half slab
 #pragma unroll
       for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
         if (j < kMma) Mma<T>::run(fb1[j & 3], fa1[j >> 2], acc[j >> 2][j & 3]);
         if (j < kSlots) {
 #pragma unroll
           for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
-            if (i < kC) { if (i == 0) copy_a_c(stage, s + 3, 0); else copy_b_c(stage, s + 3, i - 1); }
+            if (i < kC) {
+              if (i == 0) { if constexpr (GATHER) rows_of(s + 3, 0, ix); else copy_a_c(stage, s + 3, 0, 0u); }
+              else copy_b_c(stage, s + 3, i - 1);
+            }
             else read_frag_c(Next(), 0, i - kC, fa0, fb0);
           }
+          if (GATHER && kC > 0 && j == kSlots - 1) copy_a_c(stage, s + 3, 0, row_bytes(ix));
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -894,15 +941,20 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
     __builtin_amdgcn_sched_barrier(0);
     {
       constexpr int kC = C::P1 ? 3 : 0, kItems = kC + kFrags;
+      int ix[4] = {0, 0, 0, 0};  // gathered rows: the four rows of the A piece copied in this half slab
 #pragma unroll
       for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
         if (j < kMma) Mma<T>::run(fb0[j & 3], fa0[j >> 2], acc[j >> 2][j & 3]);
         if (j < kSlots) {
 #pragma unroll
           for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
-            if (i < kC) { if (i == 0) copy_a(s + 2, 1); else copy_b(s + 2, 1 + i); }
+            if (i < kC) {
+              if (i == 0) { if constexpr (GATHER) rows_of(s + 2, 1, ix); else copy_a(s + 2, 1, 0u); }
+              else copy_b(s + 2, 1 + i);
+            }
             else read_frag(s, 1, i - kC, fa1, fb1);
           }
+          if (GATHER && kC > 0 && j == kSlots - 1) copy_a(s + 2, 1, row_bytes(ix));
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -914,15 +966,20 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
     __builtin_amdgcn_sched_barrier(0);
     {
       constexpr int kC = C::P2 ? 3 : 0, kItems = kC + (C::NEXT ? kFrags : 0);
+      int ix[4] = {0, 0, 0, 0};  // gathered rows: the four rows of the A piece copied in this half slab
 #pragma unroll
       for (int j = 0; j < (kMma > 0 ? kMma : 1); ++j) {
         if (j < kMma) Mma<T>::run(fb1[j & 3], fa1[j >> 2], acc[j >> 2][j & 3]);
         if (j < kSlots) {
 #pragma unroll
           for (int i = j * kItems / kSlots; i < (j + 1) * kItems / kSlots; ++i) {
-            if (i < kC) { if (i == 0) copy_a(s + 3, 0); else copy_b(s + 3, i - 1); }
+            if (i < kC) {
+              if (i == 0) { if constexpr (GATHER) rows_of(s + 3, 0, ix); else copy_a(s + 3, 0, 0u); }
+              else copy_b(s + 3, i - 1);
+            }
             else read_frag(s + 1, 0, i - kC, fa0, fb0);
           }
+          if (GATHER && kC > 0 && j == kSlots - 1) copy_a(s + 3, 0, row_bytes(ix));
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -993,7 +1050,7 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
   }
 }
 
-template <typename T>
+template <typename T, bool GATHER>
 __global__ __launch_bounds__(kThreads, 2) void wgrad_small_kernel(const WgradArgs args) {
   const int tid = threadIdx.x, wave = tid >> 6, wm = wave >> 1;
   const int per_expert = args.n_m_tiles * args.n_n_tiles;
@@ -1012,9 +1069,9 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_small_kernel(const WgradArg
   const int n_blocks32 = (rows_m + 31) >> 5;
   const int n_mi = (n_blocks32 - wm + 1) >> 1;
   switch (n_mi) {
-    case 2: run_wgrad_tile_small<T, 2>(args, tid, expert, m0, n0, rows_m, first, rows); break;
-    case 1: run_wgrad_tile_small<T, 1>(args, tid, expert, m0, n0, rows_m, first, rows); break;
-    default: run_wgrad_tile_small<T, 0>(args, tid, expert, m0, n0, rows_m, first, rows); break;
+    case 2: run_wgrad_tile_small<T, 2, GATHER>(args, tid, expert, m0, n0, rows_m, first, rows); break;
+    case 1: run_wgrad_tile_small<T, 1, GATHER>(args, tid, expert, m0, n0, rows_m, first, rows); break;
+    default: run_wgrad_tile_small<T, 0, GATHER>(args, tid, expert, m0, n0, rows_m, first, rows); break;
   }
 }
 
@@ -1073,22 +1130,33 @@ int gemm_async_dgrad(const void *g, const int *g_rows, int g_div, const void *w,
 // their last row (the copies of a partial last slab run over; what they fetch is zeroed before use).
 bool wgrad_async_supported(int Md, int Nd) { return Md % 8 == 0 && Nd % 8 == 0; }
 
+namespace async {
+template <typename T, bool GATHER> static int launch_wgrad(const WgradArgs &a, hipStream_t stream) {
+  auto kernel = wgrad_small_kernel<T, GATHER>;
+  static DeviceFlags attr_done;  // one per kernel instantiation
+  if (int rc = ensure_dynamic_lds((const void *)kernel, kSmallLds, attr_done, "wgrad_small_kernel")) return rc;
+  long long total = (long long)a.E * a.n_m_tiles * a.n_n_tiles;
+  if (total <= 0) return 0;
+  total = (total + kXcds - 1) / kXcds * kXcds;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(kThreads), kSmallLds, stream, a);
+  return check_launch("wgrad_small_kernel");
+}
+}  // namespace async
+
+// With l_rows the left operand is not in expert order: sorted row p is row l_rows[p] / l_div of L (rows of a
+// [n_rows / l_div, Md] tensor gathered by token, which must span less than 4 GiB); l_rows holds n_rows values below
+// n_rows and must stay readable for 32 values more, and L needs no readable rows past its end.
 template <typename T>
-int gemm_async_wgrad(const void *L, const void *R, void *dW, const int *counts, const int *offsets, int capacity, int E,
-                     int Md, int Nd, hipStream_t stream) {
+int gemm_async_wgrad(const void *L, const int *l_rows, int l_div, int n_rows, const void *R, void *dW, const int *counts,
+                     const int *offsets, int capacity, int E, int Md, int Nd, hipStream_t stream) {
   async::WgradArgs a = {};
   a.A = L; a.B = R; a.C = dW; a.counts = counts; a.offsets = offsets; a.capacity = capacity;
+  a.a_rows = l_rows; a.a_div = make_fast_div(l_rows != nullptr ? l_div : 1); a.a_rows_max = n_rows > 0 ? n_rows - 1 : 0;
   a.E = E; a.Md = Md; a.Nd = Nd;
   a.n_m_tiles = ceil_div(Md, async::kSmallBM);
   a.n_n_tiles = ceil_div(Nd, async::kBN);
-  auto kernel = async::wgrad_small_kernel<T>;
-  static DeviceFlags attr_done;
-  if (int rc = ensure_dynamic_lds((const void *)kernel, async::kSmallLds, attr_done, "wgrad_small_kernel")) return rc;
-  long long total = (long long)E * a.n_m_tiles * a.n_n_tiles;
-  if (total <= 0) return 0;
-  total = (total + kXcds - 1) / kXcds * kXcds;
-  hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(async::kThreads), async::kSmallLds, stream, a);
-  return check_launch("wgrad_small_kernel");
+  if (l_rows != nullptr) return async::launch_wgrad<T, true>(a, stream);
+  return async::launch_wgrad<T, false>(a, stream);
 }
 
 #define YAMOE_INSTANTIATE_ASYNC(T)                                                                               \
@@ -1098,8 +1166,8 @@ int gemm_async_wgrad(const void *L, const void *R, void *dW, const int *counts, 
                                   int, int, hipStream_t);                                                             \
   template int gemm_async_dgrad<T>(const void *, const int *, int, const void *, void *, const void *, int, int, int,  \
                                    int, const void *, float *, hipStream_t);                                           \
-  template int gemm_async_wgrad<T>(const void *, const void *, void *, const int *, const int *, int, int, int, int,    \
-                                   hipStream_t);
+  template int gemm_async_wgrad<T>(const void *, const int *, int, int, const void *, void *, const int *, const int *, \
+                                   int, int, int, int, hipStream_t);
 YAMOE_INSTANTIATE_ASYNC(bf16_t)
 YAMOE_INSTANTIATE_ASYNC(f16_t)
 
