@@ -23,6 +23,9 @@ def test_forward_and_backward_through_ctypes_with_reused_workspace(gpu, dtype):
     cd = torch.float32 if dtype == torch.bfloat16 else torch.float64
     big = make_inputs(700, 192, 128, 8, 2, dtype, seed=61, w_std=0.05, bias_std=0.1, zipf=0.8)
     small = make_inputs(90, 192, 128, 8, 2, dtype, seed=62, w_std=0.05, bias_std=0.1)
+    # three assignments: the weight-gradient kernel's look-ups of a partial slab run past the end of the row list
+    # into whatever the workspace holds
+    tiny = make_inputs(3, 192, 128, 8, 1, dtype, seed=64, w_std=0.05, bias_std=0.1)
     # one workspace, sized for the largest call (the backward of the larger problem), poisoned before the first use
     g_big = [big[k].to(gpu) for k in KEYS]
     p = _cabi.problem(g_big[0], g_big[1], g_big[2], g_big[3], 700)
@@ -30,7 +33,7 @@ def test_forward_and_backward_through_ctypes_with_reused_workspace(gpu, dtype):
     need_b = lib.yamoe_experts_backward_workspace_bytes(ctypes.byref(p))
     assert 0 < need_f < need_b
     ws = torch.full((need_b,), 0xA5, dtype=torch.uint8, device=gpu)
-    for label, d, cap in (("big", big, 700), ("small", small, 90), ("big, capacity 50", big, 50)):
+    for label, d, cap in (("big", big, 700), ("small", small, 90), ("big, capacity 50", big, 50), ("tiny", tiny, 3)):
         print("ctypes whole op:", dtype, label, flush=True)
         g = [d[k].to(gpu) for k in KEYS]
         out = torch.full_like(g[0], float("nan"))
@@ -44,6 +47,8 @@ def test_forward_and_backward_through_ctypes_with_reused_workspace(gpu, dtype):
         torch.cuda.synchronize()
         want_g = O.experts_backward(gy, *[d[k] for k in KEYS], cap, compute_dtype=cd)
         for n, a, b in zip(NAMES, outs, want_g):
+            if label == "tiny" and n == "d_routing":
+                continue  # three entries that may cancel: pinned entry by entry in test_gpu_routing_grad.py
             assert O.rel_l2(a.cpu(), b) < tol, (label, n)
     # a workspace one byte short is refused, nothing is launched
     out = torch.zeros_like(g_big[0])
