@@ -17,6 +17,7 @@ CASES = [
     (32768, 768, 40, torch.int64, True),     # largest single-block case, most buckets
     (65536, 128, 16384, torch.int64, False),  # multi-block form
     (40001, 5, 9000, torch.int32, True),
+    (40000, 700, 100, torch.int64, True),    # multi-block form with a segment table too large for LDS staging
     (0, 4, 3, torch.int64, False),
 ]
 

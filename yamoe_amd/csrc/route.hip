@@ -361,29 +361,48 @@ __global__ __launch_bounds__(kRouteThreads) void route_hist_kernel(const void *i
     seg_counts[(size_t)blockIdx.x * kRouteWaves * buckets + i] = lds[i];
 }
 
-// One block: totals, offsets, then per-segment cursors written back over seg_counts.
-__global__ __launch_bounds__(kRouteThreads) void route_scan_kernel(int *seg_counts, int n_seg, int E,
-                                                                   int *counts, int *offsets_out) {
+// One block: totals, offsets, then per-segment cursors written back over seg_counts.  A wave takes one bucket at a time and walks its column
+// of the table 64 segments per step with a wave prefix sum.  STAGED: the table (segments x buckets) is first read into
+// LDS in one sweep and written back in another, so that all of its reads are in flight together; straight from
+// memory every step of every column is a round trip of its own (1.4 us each: 47 us for 128 segments x 129 buckets).
+constexpr int kScanStagedCells = 34816;  // 136 KB of LDS
+
+template <bool STAGED>
+__global__ __launch_bounds__(kRouteThreads) void route_scan_kernel(int *seg_counts, int n_seg, int E, int *counts,
+                                                                   int *offsets_out) {
   extern __shared__ int lds[];
   const int buckets = E + 1;
   int *total = lds;
   int *offs = total + buckets;
   int *scratch = offs + buckets + 1;
-  const int tid = threadIdx.x;
-  for (int b = tid; b < buckets; b += blockDim.x) {
+  int *staged = scratch + kRouteWaves + 1;  // [n_seg][buckets] with STAGED
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int cells = n_seg * buckets;
+  if constexpr (STAGED) {
+    for (int i = tid; i < cells; i += blockDim.x) staged[i] = seg_counts[i];
+    __syncthreads();
+  }
+  int *table = STAGED ? staged : seg_counts;
+  for (int b = wave; b < buckets; b += kRouteWaves) {
     int s = 0;
-    for (int g = 0; g < n_seg; ++g) s += seg_counts[(size_t)g * buckets + b];
-    total[b] = s;
+    for (int g = lane; g < n_seg; g += kWave) s += table[(size_t)g * buckets + b];
+    for (int d = kWave / 2; d > 0; d >>= 1) s += __shfl_xor(s, d);
+    if (lane == 0) total[b] = s;
   }
   __syncthreads();
   block_exclusive_scan(total, offs, buckets, scratch);
-  for (int b = tid; b < buckets; b += blockDim.x) {
+  for (int b = wave; b < buckets; b += kRouteWaves) {
     int run = offs[b];
-    for (int g = 0; g < n_seg; ++g) {
-      int c = seg_counts[(size_t)g * buckets + b];
-      seg_counts[(size_t)g * buckets + b] = run;
-      run += c;
+    for (int g0 = 0; g0 < n_seg; g0 += kWave) {
+      const int g = g0 + lane;
+      const int c = g < n_seg ? table[(size_t)g * buckets + b] : 0;
+      int step_total;
+      const int before = wave_exclusive_scan(c, lane, step_total);
+      if (g < n_seg) table[(size_t)g * buckets + b] = run + before;
+      run += step_total;
     }
+  }
+  for (int b = tid; b < buckets; b += blockDim.x) {
     if (b < E) {
       counts[b] = total[b];
       offsets_out[b] = offs[b];
@@ -391,15 +410,27 @@ __global__ __launch_bounds__(kRouteThreads) void route_scan_kernel(int *seg_coun
       offsets_out[E] = offs[E];
     }
   }
+  if constexpr (STAGED) {
+    __syncthreads();
+    for (int i = tid; i < cells; i += blockDim.x) seg_counts[i] = staged[i];
+  }
 }
 
+// With sched the grid has one workgroup more than there are blocks of segments: its first wave writes the work lists
+// of the GEMM kernels from the counts and offsets, next to the placement instead of in a launch of its own.
 template <bool I64>
 __global__ __launch_bounds__(kRouteThreads) void route_place_kernel(
     const void *idx, int N, int E, int capacity, int seg, const int *seg_cursors,
-    const int *offsets_in, int *sorted_expert, int *sorted_idx, int *inv_pos) {
+    const int *offsets_in, int *sorted_expert, int *sorted_idx, int *inv_pos, int n_blocks, const int *counts,
+    int stream_max_rows, int *sched) {
   extern __shared__ int lds[];
   const int buckets = E + 1;
   const int tid = threadIdx.x, wave = tid / kWave;
+  if ((int)blockIdx.x >= n_blocks) {  // (uniform for the workgroup: nobody of it reaches the barrier below)
+    if (sched != nullptr && wave == 0)
+      build_schedule_wave(counts, offsets_in, N, E, capacity, stream_max_rows, sched, tid);
+    return;
+  }
   int *cursor = lds + wave * buckets;
   int *offs = lds + kRouteWaves * buckets;
   for (int i = tid; i < kRouteWaves * buckets; i += blockDim.x)
@@ -416,15 +447,21 @@ __global__ __launch_bounds__(kRouteThreads) void route_place_kernel(
 
 using namespace yamoe;
 
+// Keys per wave in the three-kernel form: short segments spread the counting and the placement over more workgroups,
+// long ones keep the scan's table (segments x buckets, walked by one workgroup) small.  65 536 keys, 128 experts:
+// 46 / 40 / 48 us for the three launches with segments of 1024 / 512 / 256 keys (85 us with 2048 and the work lists in a
+// launch of their own).
+static int route_segment(int N) { return N <= 4 * kSingleBlockMaxN ? 512 : 2048; }
+
 extern "C" size_t yamoe_route_workspace_bytes(int32_t N, int32_t E) {
   if (N <= kSingleBlockMaxN) return 256;
-  int seg = 2048;
+  int seg = route_segment(N);
   int n_seg = ceil_div(ceil_div(N, seg), kRouteWaves) * kRouteWaves;
   return align_up((size_t)n_seg * (E + 1) * sizeof(int), 256);
 }
 
-// yamoe_route, optionally followed by yamoe_build_schedule (schedule != nullptr); for N up to kSingleBlockMaxN both
-// run in one launch.
+// yamoe_route, optionally with the work lists of yamoe_build_schedule (schedule != nullptr): one launch for N up to
+// kSingleBlockMaxN, three above (the lists come from an extra workgroup of the placement kernel).
 int yamoe::route_and_schedule(const void *router_indices, int32_t idx_i64, int32_t N, int32_t E, int32_t capacity,
                               int32_t *sorted_expert, int32_t *sorted_idx, int32_t *counts, int32_t *offsets,
                               int32_t *inv_pos, void *workspace, size_t workspace_bytes, int32_t stream_max_rows,
@@ -467,7 +504,7 @@ int yamoe::route_and_schedule(const void *router_indices, int32_t idx_i64, int32
     set_error("yamoe_route: workspace too small (%zu < %zu)", workspace_bytes, yamoe_route_workspace_bytes(N, E));
     return YAMOE_E_WORKSPACE;
   }
-  const int seg = 2048;
+  const int seg = route_segment(N);
   const int n_blocks = ceil_div(ceil_div(N, seg), kRouteWaves);
   const int n_seg = n_blocks * kRouteWaves;
   int *seg_counts = (int *)workspace;
@@ -482,19 +519,28 @@ int yamoe::route_and_schedule(const void *router_indices, int32_t idx_i64, int32
                        router_indices, N, E, seg, seg_counts);
   int rc = check_launch("route_hist_kernel");
   if (rc) return rc;
-  hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(kRouteThreads), lds_b, stream, seg_counts, n_seg, E,
-                     counts, offsets);
+  if ((long long)n_seg * buckets <= kScanStagedCells) {
+    static DeviceFlags attr_scan;
+    const int max_lds = (int)(((size_t)kRouteMaxBuckets * 2 + 1 + kRouteWaves + 1 + kScanStagedCells) * sizeof(int));
+    rc = ensure_dynamic_lds((const void *)route_scan_kernel<true>, max_lds, attr_scan, "route_scan_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL(route_scan_kernel<true>, dim3(1), dim3(kRouteThreads), lds_b + (size_t)n_seg * buckets * sizeof(int),
+                       stream, seg_counts, n_seg, E, counts, offsets);
+  } else {
+    hipLaunchKernelGGL(route_scan_kernel<false>, dim3(1), dim3(kRouteThreads), lds_b, stream, seg_counts, n_seg, E, counts,
+                       offsets);
+  }
   rc = check_launch("route_scan_kernel");
   if (rc) return rc;
   if (idx_i64)
-    hipLaunchKernelGGL(route_place_kernel<true>, dim3(n_blocks), dim3(kRouteThreads), lds_c, stream,
-                       router_indices, N, E, capacity, seg, seg_counts, offsets, sorted_expert, sorted_idx, inv_pos);
+    hipLaunchKernelGGL(route_place_kernel<true>, dim3(n_blocks + (schedule != nullptr ? 1 : 0)), dim3(kRouteThreads), lds_c,
+                       stream, router_indices, N, E, capacity, seg, seg_counts, offsets, sorted_expert, sorted_idx, inv_pos,
+                       n_blocks, counts, stream_max_rows, (int *)schedule);
   else
-    hipLaunchKernelGGL(route_place_kernel<false>, dim3(n_blocks), dim3(kRouteThreads), lds_c, stream,
-                       router_indices, N, E, capacity, seg, seg_counts, offsets, sorted_expert, sorted_idx, inv_pos);
-  rc = check_launch("route_place_kernel");
-  if (rc || schedule == nullptr) return rc;
-  return yamoe_build_schedule(counts, offsets, N, E, capacity, stream_max_rows, schedule, schedule_bytes, stream_);
+    hipLaunchKernelGGL(route_place_kernel<false>, dim3(n_blocks + (schedule != nullptr ? 1 : 0)), dim3(kRouteThreads), lds_c,
+                       stream, router_indices, N, E, capacity, seg, seg_counts, offsets, sorted_expert, sorted_idx, inv_pos,
+                       n_blocks, counts, stream_max_rows, (int *)schedule);
+  return check_launch("route_place_kernel");
 }
 
 extern "C" int yamoe_route(const void *router_indices, int32_t idx_i64, int32_t N, int32_t E,
