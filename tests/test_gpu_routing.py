@@ -19,6 +19,12 @@ CASES = [
     (40001, 5, 9000, torch.int32, True),
     (40000, 700, 100, torch.int64, True),    # multi-block form with a segment table too large for LDS staging
     (0, 4, 3, torch.int64, False),
+    # either side of the sizes at which the form changes (one workgroup / two launches / other segment lengths)
+    (4096, 16, 300, torch.int64, True),
+    (4097, 16, 300, torch.int32, True),
+    (32768, 64, 500, torch.int64, False),
+    (32769, 64, 500, torch.int32, True),
+    (131073, 9, 20000, torch.int64, True),
 ]
 
 

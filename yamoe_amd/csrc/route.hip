@@ -16,7 +16,8 @@ namespace yamoe {
 constexpr int kRouteThreads = 1024;
 constexpr int kRouteWaves = kRouteThreads / kWave;
 constexpr int kRouteMaxBuckets = 769;    // E + 1 must not exceed this (keeps dynamic LDS under 64 KB)
-constexpr int kSingleBlockMaxN = 32768;  // above this the three-kernel form is used
+constexpr int kSingleBlockMaxN = 32768;  // the single-workgroup kernel's limit (its keys sit in LDS as 16-bit values)
+constexpr int kSingleBlockN = 4096;      // up to this many assignments the single-workgroup kernel is used
 
 template <bool I64>
 __device__ inline int load_key(const void *idx, int i, int E) {
@@ -361,13 +362,10 @@ __global__ __launch_bounds__(kRouteThreads) void route_hist_kernel(const void *i
     seg_counts[(size_t)blockIdx.x * kRouteWaves * buckets + i] = lds[i];
 }
 
-// One block: totals, offsets, then per-segment cursors written back over seg_counts.  A wave takes one bucket at a time and walks its column
-// of the table 64 segments per step with a wave prefix sum.  STAGED: the table (segments x buckets) is first read into
-// LDS in one sweep and written back in another, so that all of its reads are in flight together; straight from
-// memory every step of every column is a round trip of its own (1.4 us each: 47 us for 128 segments x 129 buckets).
-constexpr int kScanStagedCells = 34816;  // 136 KB of LDS
-
-template <bool STAGED>
+// One block: totals, offsets, then per-segment cursors written back over seg_counts.  A wave takes one bucket at a
+// time and walks its column of the table 64 segments per step with a wave prefix sum.  Every step is a round trip to
+// memory (1.4 us): this is the form for tables too large for LDS (many experts and many assignments at once);
+// smaller ones take route_place_scan_kernel.
 __global__ __launch_bounds__(kRouteThreads) void route_scan_kernel(int *seg_counts, int n_seg, int E, int *counts,
                                                                    int *offsets_out) {
   extern __shared__ int lds[];
@@ -375,17 +373,10 @@ __global__ __launch_bounds__(kRouteThreads) void route_scan_kernel(int *seg_coun
   int *total = lds;
   int *offs = total + buckets;
   int *scratch = offs + buckets + 1;
-  int *staged = scratch + kRouteWaves + 1;  // [n_seg][buckets] with STAGED
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-  const int cells = n_seg * buckets;
-  if constexpr (STAGED) {
-    for (int i = tid; i < cells; i += blockDim.x) staged[i] = seg_counts[i];
-    __syncthreads();
-  }
-  int *table = STAGED ? staged : seg_counts;
   for (int b = wave; b < buckets; b += kRouteWaves) {
     int s = 0;
-    for (int g = lane; g < n_seg; g += kWave) s += table[(size_t)g * buckets + b];
+    for (int g = lane; g < n_seg; g += kWave) s += seg_counts[(size_t)g * buckets + b];
     for (int d = kWave / 2; d > 0; d >>= 1) s += __shfl_xor(s, d);
     if (lane == 0) total[b] = s;
   }
@@ -395,10 +386,10 @@ __global__ __launch_bounds__(kRouteThreads) void route_scan_kernel(int *seg_coun
     int run = offs[b];
     for (int g0 = 0; g0 < n_seg; g0 += kWave) {
       const int g = g0 + lane;
-      const int c = g < n_seg ? table[(size_t)g * buckets + b] : 0;
+      const int c = g < n_seg ? seg_counts[(size_t)g * buckets + b] : 0;
       int step_total;
       const int before = wave_exclusive_scan(c, lane, step_total);
-      if (g < n_seg) table[(size_t)g * buckets + b] = run + before;
+      if (g < n_seg) seg_counts[(size_t)g * buckets + b] = run + before;
       run += step_total;
     }
   }
@@ -409,10 +400,6 @@ __global__ __launch_bounds__(kRouteThreads) void route_scan_kernel(int *seg_coun
     } else {
       offsets_out[E] = offs[E];
     }
-  }
-  if constexpr (STAGED) {
-    __syncthreads();
-    for (int i = tid; i < cells; i += blockDim.x) seg_counts[i] = staged[i];
   }
 }
 
@@ -443,25 +430,90 @@ __global__ __launch_bounds__(kRouteThreads) void route_place_kernel(
                   inv_pos);
 }
 
+// ---- two-kernel form: every workgroup of the placement scans the table for itself -----------------------------
+// The segments x buckets table of route_hist_kernel is small (65 536 keys in segments of 512 and 128 experts: 66 KB),
+// so instead of one workgroup scanning it in a launch of its own, every workgroup of the placement reads all of it
+// into LDS and derives what it needs: the bucket totals and offsets, and the cursors of its own 16 segments (a wave
+// per bucket column, wave prefix sums over the segments).  Workgroup 0 also writes counts and offsets; with sched
+// one workgroup more than there are blocks of segments writes the work lists.
+__host__ __device__ inline size_t route_place_scan_lds_ints(int n_seg, int buckets) {
+  return (size_t)buckets + (buckets + 1) + (kRouteWaves + 1) + (size_t)kRouteWaves * buckets + (size_t)n_seg * buckets;
+}
+constexpr size_t kPlaceScanMaxLdsInts = 40000;  // 160 000 bytes
+
+template <bool I64>
+__global__ __launch_bounds__(kRouteThreads) void route_place_scan_kernel(
+    const void *idx, int N, int E, int capacity, int seg, const int *seg_counts, int n_seg, int *sorted_expert,
+    int *sorted_idx, int *inv_pos, int *counts, int *offsets_out, int n_blocks, int stream_max_rows, int *sched) {
+  extern __shared__ int lds[];
+  const int buckets = E + 1;
+  int *total = lds;                              // [buckets]
+  int *offs = total + buckets;                   // [buckets + 1]
+  int *scratch = offs + buckets + 1;             // [kRouteWaves + 1]
+  int *cursors = scratch + kRouteWaves + 1;      // [kRouteWaves][buckets]
+  int *table = cursors + kRouteWaves * buckets;  // [n_seg][buckets]
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int cells = n_seg * buckets;
+  for (int i = tid; i < cells; i += blockDim.x) table[i] = seg_counts[i];
+  __syncthreads();
+  const int my_first = blockIdx.x * kRouteWaves;  // this workgroup's segments: my_first + 0..15 (none for the extra one)
+  for (int b = wave; b < buckets; b += kRouteWaves) {
+    int run = 0;
+    for (int g0 = 0; g0 < n_seg; g0 += kWave) {
+      const int g = g0 + lane;
+      const int c = g < n_seg ? table[g * buckets + b] : 0;
+      int step_total;
+      const int before = wave_exclusive_scan(c, lane, step_total);
+      if (g < n_seg && g >= my_first && g < my_first + kRouteWaves) cursors[(g - my_first) * buckets + b] = run + before;
+      run += step_total;
+    }
+    if (lane == 0) total[b] = run;
+  }
+  __syncthreads();
+  block_exclusive_scan(total, offs, buckets, scratch);
+  if (blockIdx.x == 0) {
+    for (int b = tid; b < buckets; b += blockDim.x) {
+      if (b < E) {
+        counts[b] = total[b];
+        offsets_out[b] = offs[b];
+      } else {
+        offsets_out[E] = offs[E];
+      }
+    }
+  }
+  if ((int)blockIdx.x >= n_blocks) {  // (uniform for the workgroup: nobody of it reaches the barrier below)
+    if (sched != nullptr && wave == 0) build_schedule_wave(total, offs, N, E, capacity, stream_max_rows, sched, lane);
+    return;
+  }
+  for (int i = tid; i < kRouteWaves * buckets; i += blockDim.x) cursors[i] += offs[i % buckets];
+  __syncthreads();
+  const int sgm = my_first + wave;
+  const int seg_begin = (int)min((long long)sgm * seg, (long long)N), seg_end = min(seg_begin + seg, N);
+  wave_place<I64>(idx, seg_begin, seg_end, E, capacity, cursors + wave * buckets, offs, sorted_expert, sorted_idx, inv_pos);
+}
+
 }  // namespace yamoe
 
 using namespace yamoe;
 
-// Keys per wave in the three-kernel form: short segments spread the counting and the placement over more workgroups,
-// long ones keep the scan's table (segments x buckets, walked by one workgroup) small.  65 536 keys, 128 experts:
-// 46 / 40 / 48 us for the three launches with segments of 1024 / 512 / 256 keys (85 us with 2048 and the work lists in a
-// launch of their own).
-static int route_segment(int N) { return N <= 4 * kSingleBlockMaxN ? 512 : 2048; }
+// Keys per wave in the forms with more than one launch: short segments spread the counting and the placement over
+// more workgroups, long ones keep the segments x buckets table small.  65 536 keys, 128 experts, three launches:
+// 46 / 40 / 48 us with segments of 1024 / 512 / 256 keys (85 us with 2048 and the work lists in a launch of their own),
+// two launches with 512: 33 us.  16 384 keys, 32 experts, two launches: 20.5 / 16.3 / 18 us with 512 / 256 / 128 against
+// 26 us for the single-workgroup kernel.
+static int route_segment(int N) { return N <= 32768 ? 256 : N <= 131072 ? 512 : 2048; }
+static_assert(kSingleBlockN <= kSingleBlockMaxN, "the single-workgroup kernel keeps its keys in LDS");
 
 extern "C" size_t yamoe_route_workspace_bytes(int32_t N, int32_t E) {
-  if (N <= kSingleBlockMaxN) return 256;
+  if (N <= kSingleBlockN) return 256;
   int seg = route_segment(N);
   int n_seg = ceil_div(ceil_div(N, seg), kRouteWaves) * kRouteWaves;
   return align_up((size_t)n_seg * (E + 1) * sizeof(int), 256);
 }
 
 // yamoe_route, optionally with the work lists of yamoe_build_schedule (schedule != nullptr): one launch for N up to
-// kSingleBlockMaxN, three above (the lists come from an extra workgroup of the placement kernel).
+// kSingleBlockN, two above (histograms, then scan + placement), three where the histogram table does not fit LDS;
+// with more than one launch the lists come from an extra workgroup of the placement kernel.
 int yamoe::route_and_schedule(const void *router_indices, int32_t idx_i64, int32_t N, int32_t E, int32_t capacity,
                               int32_t *sorted_expert, int32_t *sorted_idx, int32_t *counts, int32_t *offsets,
                               int32_t *inv_pos, void *workspace, size_t workspace_bytes, int32_t stream_max_rows,
@@ -483,7 +535,7 @@ int yamoe::route_and_schedule(const void *router_indices, int32_t idx_i64, int32
   }
   if (capacity < 0) capacity = 0;
   const int buckets = E + 1;
-  if (N <= kSingleBlockMaxN) {
+  if (N <= kSingleBlockN) {
     size_t lds = route_single_lds_bytes(N, buckets);
     static DeviceFlags attr_i64, attr_i32;
     const int max_lds = (int)route_single_lds_bytes(kSingleBlockMaxN, kRouteMaxBuckets);
@@ -519,17 +571,26 @@ int yamoe::route_and_schedule(const void *router_indices, int32_t idx_i64, int32
                        router_indices, N, E, seg, seg_counts);
   int rc = check_launch("route_hist_kernel");
   if (rc) return rc;
-  if ((long long)n_seg * buckets <= kScanStagedCells) {
-    static DeviceFlags attr_scan;
-    const int max_lds = (int)(((size_t)kRouteMaxBuckets * 2 + 1 + kRouteWaves + 1 + kScanStagedCells) * sizeof(int));
-    rc = ensure_dynamic_lds((const void *)route_scan_kernel<true>, max_lds, attr_scan, "route_scan_kernel");
+  if (route_place_scan_lds_ints(n_seg, buckets) <= kPlaceScanMaxLdsInts) {
+    // two launches: the placement's workgroups scan the table themselves
+    static DeviceFlags attr_ps64, attr_ps32;
+    const int max_lds = (int)(kPlaceScanMaxLdsInts * sizeof(int));
+    rc = idx_i64 ? ensure_dynamic_lds((const void *)route_place_scan_kernel<true>, max_lds, attr_ps64, "route_place_scan_kernel")
+                 : ensure_dynamic_lds((const void *)route_place_scan_kernel<false>, max_lds, attr_ps32, "route_place_scan_kernel");
     if (rc) return rc;
-    hipLaunchKernelGGL(route_scan_kernel<true>, dim3(1), dim3(kRouteThreads), lds_b + (size_t)n_seg * buckets * sizeof(int),
-                       stream, seg_counts, n_seg, E, counts, offsets);
-  } else {
-    hipLaunchKernelGGL(route_scan_kernel<false>, dim3(1), dim3(kRouteThreads), lds_b, stream, seg_counts, n_seg, E, counts,
-                       offsets);
+    const size_t lds_ps = route_place_scan_lds_ints(n_seg, buckets) * sizeof(int);
+    const dim3 grid(n_blocks + (schedule != nullptr ? 1 : 0));
+    if (idx_i64)
+      hipLaunchKernelGGL(route_place_scan_kernel<true>, grid, dim3(kRouteThreads), lds_ps, stream, router_indices, N, E,
+                         capacity, seg, seg_counts, n_seg, sorted_expert, sorted_idx, inv_pos, counts, offsets, n_blocks,
+                         stream_max_rows, (int *)schedule);
+    else
+      hipLaunchKernelGGL(route_place_scan_kernel<false>, grid, dim3(kRouteThreads), lds_ps, stream, router_indices, N, E,
+                         capacity, seg, seg_counts, n_seg, sorted_expert, sorted_idx, inv_pos, counts, offsets, n_blocks,
+                         stream_max_rows, (int *)schedule);
+    return check_launch("route_place_scan_kernel");
   }
+  hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(kRouteThreads), lds_b, stream, seg_counts, n_seg, E, counts, offsets);
   rc = check_launch("route_scan_kernel");
   if (rc) return rc;
   if (idx_i64)
