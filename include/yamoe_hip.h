@@ -23,7 +23,9 @@
 extern "C" {
 #endif
 
-#define YAMOE_ABI_VERSION 1
+/* 2: YAMOE_F64 dtype code; yamoe_experts_forward_static; yamoe_route_workspace_bytes returns the size of a
+ *    segments x buckets table above 4096 assignments (it was a constant 256 bytes); stream_max_rows up to 32. */
+#define YAMOE_ABI_VERSION 2
 
 /* element type of activations, weights, biases and routing weights.  YAMOE_F64 is taken by the row movers among
  * the helper ops only (yamoe_padded_gather, yamoe_padded_scatter, yamoe_index_select), which the reference

@@ -327,26 +327,29 @@ def batch_mm(x, weights, compute_dtype=torch.float64):
 # ------------------------------------------------------------------------------------------------
 # router step
 # ------------------------------------------------------------------------------------------------
-def router_from_logits(logits, top_k):
+def router_from_logits(logits, top_k, compute_dtype=torch.float32, picks=None):
     """top-k -> softmax over the picked logits -> dense scores (torch-ext/yamoe/layers.py:135-152,
     torch-ext/yamoe/vendored/gpt_oss_mlp.py:134-142).  Picks come in descending order of logit; among equal
-    logits the lower expert id first (torch.topk leaves that order open).  The softmax is taken in fp32 and
-    rounded once to the logits' dtype.  Returns (router_indices int64 [T,K], router_scores [T,E])."""
-    order = torch.sort(logits.float(), dim=-1, descending=True, stable=True).indices[:, :top_k]
-    top = torch.gather(logits.float(), 1, order)
+    logits the lower expert id first (torch.topk leaves that order open).  The softmax is taken in
+    `compute_dtype` and rounded once to the logits' dtype.  `picks` (int64 [T,K]) replaces the top-k when the
+    caller already knows which experts were chosen (a gradient check on somebody else's routing); the rest is
+    differentiable with respect to the logits.  Returns (router_indices int64 [T,K], router_scores [T,E])."""
+    lg = logits.to(compute_dtype)
+    order = picks if picks is not None else torch.sort(lg.detach(), dim=-1, descending=True, stable=True).indices[:, :top_k]
+    top = torch.gather(lg, 1, order)
     w = torch.softmax(top, dim=-1).to(logits.dtype)
-    scores = torch.zeros_like(logits).scatter_(1, order, w)
+    scores = torch.zeros_like(logits).scatter(1, order, w)
     return order, scores
 
 
-def router(hidden, weight, bias, top_k):
-    """logits = hidden . weight^T + bias in fp32, rounded to the activation dtype (the output of the reference's
-    F.linear, layers.py:130-132), then router_from_logits.  Returns (indices, scores, logits)."""
-    logits = hidden.float() @ weight.float().t()
+def router(hidden, weight, bias, top_k, compute_dtype=torch.float32, picks=None):
+    """logits = hidden . weight^T + bias in `compute_dtype`, rounded to the activation dtype (the output of the
+    reference's F.linear, layers.py:130-132), then router_from_logits.  Returns (indices, scores, logits)."""
+    logits = hidden.to(compute_dtype) @ weight.to(compute_dtype).t()
     if bias is not None:
-        logits = logits + bias.float()
+        logits = logits + bias.to(compute_dtype)
     logits = logits.to(hidden.dtype)
-    idx, scores = router_from_logits(logits, top_k)
+    idx, scores = router_from_logits(logits, top_k, compute_dtype, picks)
     return idx, scores, logits
 
 

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), n
     assert sorted(_cabi.SYMBOLS) == names
-    assert lib.yamoe_abi_version() == 1
+    assert lib.yamoe_abi_version() == _cabi.ABI_VERSION == 2
 
 
 def test_size_queries_and_validation_need_no_gpu():

@@ -9,7 +9,7 @@ from yamoe_amd.workloads import make_config, make_inputs
 pytestmark = pytest.mark.gpu
 
 NAMES = ("d_hidden", "d_routing", "d_gate_up_proj", "d_gate_up_proj_bias", "d_down_proj", "d_down_proj_bias")
-TOL = {torch.float32: 2e-5, torch.bfloat16: 1e-2, torch.float16: 1e-2}
+TOL = {torch.float32: 1e-5, torch.bfloat16: 1e-2, torch.float16: 1e-2}
 
 
 def run_bwd(d, gy, capacity, gpu):
@@ -193,3 +193,48 @@ def test_stored_pre_activations_keep_the_clamp_decision(gpu, dtype, T):
     assert torch.all(gate_g[gate_w < 7 - margin] <= 7) and torch.all(up_g[up_w.abs() < 7 - margin].abs() <= 7)
     inside = want.abs() < 6.9
     assert float((got[inside] - want[inside]).abs().max()) < 0.04  # (within a rounding step of the fp64 value)
+
+
+def test_backward_fp32_pre_activation_on_the_clamp_boundary(gpu):
+    """The gradient of the clamp jumps at +-7 (csrc/experts_backward.cu:285-299), so a pre-activation within fp32
+    accumulation error of the limit may fall on one side on the GPU and on the other in the oracle's fp64.  This seeded
+    case has exactly one such value among its 1.2 million (an up value of -6.9999988 in fp64).  What the contract allows
+    there: the forward still agrees to 1e-5; gradients that do not pass through the clamp agree to 1e-5; the others
+    agree to 1e-5 everywhere except in the entries that one pre-activation feeds (its token's row of d_hidden, its
+    column of the expert's d_gate_up_proj and d_gate_up_proj_bias), and to 5e-3 with those entries counted."""
+    import numpy as np
+    import yamoe_amd
+    T, H, I, E, K, cap = 1025, 280, 240, 7, 5, 366
+    d = make_inputs(T, H, I, E, K, torch.float32, seed=1005, w_std=1.0, bias_std=0.1, zipf=1.2)
+    d["routing_weights"] = torch.gather(d["routing_weights"], 1, d["router_indices"])
+    gy = torch.randn(T, H, generator=torch.Generator().manual_seed(6))
+    g = to_dev(d, gpu)
+    out = yamoe_amd.experts(*args(g), cap, E, K)
+    grads = run_bwd(d, gy, cap, gpu)
+    want_out = O.experts_capacity(*args(d), cap, compute_dtype=torch.float64)
+    want = O.experts_backward(gy, *args(d), cap, compute_dtype=torch.float64)
+    assert O.rel_l2(out.cpu(), want_out) < 1e-5
+    # the pre-activations of the kept rows in fp64 that lie within 2e-5 of a clamp limit
+    r = O.route(d["router_indices"].numpy(), E, cap)
+    x, W, Bs = d["hidden"].double(), d["gate_up_proj"].double(), d["gate_up_proj_bias"].double()
+    near = []
+    for e in range(E):
+        kept, first = min(int(r["counts"][e]), cap), int(r["offsets"][e])
+        toks = torch.from_numpy(r["sorted_idx"][first:first + kept].astype(np.int64)) // K
+        pre = x[toks] @ W[e] + Bs[e]
+        close = (pre.abs() - 7).abs() < 2e-5
+        close[:, 0::2] &= pre[:, 0::2] > 0            # the gate half is clamped from above only
+        near += [(e, int(toks[i]), int(c)) for i, c in close.nonzero().tolist()]
+    print("pre-activations on the boundary:", near, flush=True)
+    assert len(near) == 1
+    e, tok, col = near[0]
+    rel = {n: O.rel_l2(a, b) for n, a, b in zip(NAMES, grads, want)}
+    print({n: "%.2e" % v for n, v in rel.items()}, flush=True)
+    for n in ("d_routing", "d_down_proj", "d_down_proj_bias"):
+        assert rel[n] < 1e-5, (n, rel[n])
+    fed = {"d_hidden": (tok, slice(None)), "d_gate_up_proj": (e, slice(None), col), "d_gate_up_proj_bias": (e, col)}
+    for n, where in fed.items():
+        a, b = grads[NAMES.index(n)].clone().double(), want[NAMES.index(n)].double()
+        assert rel[n] < 5e-3, (n, rel[n])
+        a[where] = b[where]
+        assert O.rel_l2(a, b) < 1e-5, (n, "outside the entries fed by the boundary value", O.rel_l2(a, b))

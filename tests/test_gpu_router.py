@@ -146,3 +146,41 @@ def test_yamoe_layer_reference_capacity_and_timing(gpu, dtype):
     with torch.no_grad():
         out2, _ = yamoe_amd.Yamoe.forward(dev, x.to(gpu))
     assert report("layer, no drop", out2.cpu().reshape(-1, H).double(), full, tol) < tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_yamoe_layer_trains_the_router(gpu, dtype):
+    """enable_router_grads = True survives the call (the reference resets it, torch-ext/yamoe/layers.py:110, so its
+    router never trains) and loss.backward() through the layer reaches the router's weight and bias, the hidden
+    states and the expert parameters with the gradients autograd gives through the oracle's router step and expert
+    layer on the layer's own picks."""
+    import yamoe_amd
+    B, S, H, I, E, K = 2, 96, 128, 64, 8, 2
+    blk = Block(H, I, E, K, dtype, 24)
+    x = torch.randn(B, S, H, generator=torch.Generator().manual_seed(25)).to(dtype)
+    gy = torch.randn(B, S, H, generator=torch.Generator().manual_seed(26)).to(dtype)
+    dev = Block(H, I, E, K, dtype, 24).to(gpu)
+    dev.enable_router_grads = True
+    xd = x.to(gpu).requires_grad_(True)
+    out, scores = yamoe_amd.Yamoe.forward(dev, xd)
+    assert dev.enable_router_grads is True
+    assert out.requires_grad and scores.requires_grad
+    (out * gy.to(gpu)).sum().backward()
+    torch.cuda.synchronize()
+    picks = torch.topk(scores.detach().float().cpu(), K, dim=-1).indices
+    cd = torch.float64 if dtype == torch.float32 else torch.float32
+    params = [blk.router.weight, blk.router.bias, blk.experts.gate_up_proj, blk.experts.gate_up_proj_bias,
+              blk.experts.down_proj, blk.experts.down_proj_bias]
+    leaves = [t.detach().to(cd).requires_grad_(True) for t in [x.reshape(-1, H)] + [p.data for p in params]]
+    _, want_scores, _ = O.router(leaves[0], leaves[1], leaves[2], K, compute_dtype=cd, picks=picks)
+    want_out = O.experts_capacity(leaves[0], picks, want_scores, *leaves[3:], B * S, compute_dtype=cd)
+    want = torch.autograd.grad(want_out, leaves, gy.reshape(-1, H).to(cd))
+    tol = REL_L2_TOL[dtype] if dtype == torch.float32 else 2e-2   # bf16: scores and logits are rounded along the chain
+    assert report("layer out", out.detach().cpu().reshape(-1, H).double(), want_out.detach(), tol) < tol
+    got = [xd.grad.reshape(-1, H), dev.router.weight.grad, dev.router.bias.grad, dev.experts.gate_up_proj.grad,
+           dev.experts.gate_up_proj_bias.grad, dev.experts.down_proj.grad, dev.experts.down_proj_bias.grad]
+    names = ("d_hidden", "d_router_weight", "d_router_bias", "d_gate_up_proj", "d_gate_up_proj_bias", "d_down_proj",
+             "d_down_proj_bias")
+    for n, a, b in zip(names, got, want):
+        assert a is not None, n
+        assert report("router training " + n, a.cpu().double(), b.double(), tol) < tol, n

@@ -338,3 +338,17 @@ def test_router_linear_rounds_once():
     want = (x.double() @ w.double().t() + b.double()).to(torch.bfloat16)
     assert logits.dtype == torch.bfloat16 and (logits.float() - want.float()).abs().max() <= 2 ** -7 * want.float().abs().max()
     assert idx.shape == (7, 2) and scores.shape == (7, 5)
+
+
+def test_router_is_differentiable_and_picks_override():
+    """The router step in fp64 passes a finite-difference gradient check with respect to hidden states, weight and
+    bias (the top-k choice is held fixed by the perturbation size), and `picks` reproduces the scores of the
+    step's own choice."""
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(6, 10, generator=g, dtype=torch.float64, requires_grad=True)
+    w = torch.randn(5, 10, generator=g, dtype=torch.float64, requires_grad=True)
+    b = torch.randn(5, generator=g, dtype=torch.float64, requires_grad=True)
+    idx, scores, _ = O.router(x, w, b, 3, compute_dtype=torch.float64)
+    idx2, scores2, _ = O.router(x, w, b, 3, compute_dtype=torch.float64, picks=idx)
+    assert torch.equal(idx, idx2) and torch.equal(scores, scores2)
+    assert torch.autograd.gradcheck(lambda a, c, d: O.router(a, c, d, 3, compute_dtype=torch.float64, picks=idx)[1], (x, w, b))

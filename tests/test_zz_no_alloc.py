@@ -2,7 +2,12 @@
 
 It runs the kernels of yamoe_experts_forward on a different workspace address, so its output must equal that entry
 point's bit for bit; checked on two calls in a row, the second on a smaller problem (the array then still holds the
-first call's lists and rows), and once more after the first problem again.  Problems beyond the array are refused."""
+first call's lists and rows), and once more after the first problem again.  Problems beyond the array are refused.
+
+"Allocates nothing" is checked at two levels: torch's caching allocator sees no request, and the driver's count of
+free device memory (hipMemGetInfo, which a hipMalloc or hipFree inside the library would move, whoever made it) is
+the same before and after every call but the first on the device (that one may load the code object that holds the
+array).  A hipMalloc inside the call would also make the stream capture of the last test fail."""
 import ctypes
 
 import pytest
@@ -19,10 +24,14 @@ def both(d, capacity, gpu):
     g = [d[k].to(gpu) for k in KEYS]
     want = _cabi.experts_forward(*g, capacity)
     got = torch.full_like(want, float("nan"))
-    before = torch.cuda.memory_allocated()
-    _cabi.experts_forward_static(*g, capacity, got)
-    assert torch.cuda.memory_allocated() == before
+    _cabi.experts_forward_static(*g, capacity, got)     # (the first call on the device looks the array's address up)
     torch.cuda.synchronize()
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
+    got.fill_(float("nan"))
+    _cabi.experts_forward_static(*g, capacity, got)
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before, "device memory was allocated or freed during the call"
     return got.cpu(), want.cpu()
 
 

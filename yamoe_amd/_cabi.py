@@ -12,6 +12,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libyamoe_hip.so")
 
+ABI_VERSION = 2   # YAMOE_ABI_VERSION of the header this module mirrors
 F32, F16, BF16 = 0, 1, 2
 _DTYPE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 
@@ -42,6 +43,9 @@ def lib():
         L = ctypes.CDLL(LIB_PATH)
         vp, i32, sz = ctypes.c_void_p, ctypes.c_int32, ctypes.c_size_t
         L.yamoe_abi_version.restype = ctypes.c_int
+        if L.yamoe_abi_version() != ABI_VERSION:
+            raise ImportError("%s has ABI version %d, this binding was written for %d: rebuild with `python -m yamoe_amd.build`"
+                              % (LIB_PATH, L.yamoe_abi_version(), ABI_VERSION))
         L.yamoe_last_error.restype = ctypes.c_char_p
         L.yamoe_route_workspace_bytes.restype = sz
         L.yamoe_route_workspace_bytes.argtypes = [i32, i32]

@@ -71,6 +71,7 @@ class Yamoe(torch.nn.Module):
         top_k = getattr(self, "top_k", 4)
         timing = getattr(self, "_timing_enabled", False)
         stats = {}
+        self._timing_stats = stats   # reset on every call, like the reference's (layers.py:119-122)
 
         def lap(name, since):
             torch.cuda.synchronize()
@@ -110,6 +111,9 @@ class Yamoe(torch.nn.Module):
         elif capacity == "reference":
             capacity = (tokens * top_k + num_experts - 1) // num_experts
         capacity = int(capacity)
+        if timing:
+            t1 = lap("setup", t1)    # weight slices and capacity: outside "experts_kernel", as in layers.py:158-165
+            del stats["setup"]
         if want_router_grads:
             out = experts_autograd(x_flat, router_indices, router_scores, gate_up, gate_up_bias,
                                    self.experts.down_proj, self.experts.down_proj_bias, capacity, num_experts, top_k,
@@ -121,5 +125,4 @@ class Yamoe(torch.nn.Module):
         if timing:
             lap("experts_kernel", t1)
             lap("total", t0)
-            self._timing_stats = stats
         return out.view(batch, seq, hidden), router_scores
