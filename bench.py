@@ -18,7 +18,9 @@ Also on the line:
   parity        the timed op's output against that oracle run
   configs       all five measured workloads, each with its time, its rate against its own peak (fp32 or bf16
                 MFMA, HBM for the decode shape) and its parity against the oracle:
-                cfg1 README shape fp32, cfg2 the headline, cfg3 decode, cfg4 Zipf-skewed, cfg5 backward
+                cfg1 README shape fp32, cfg2 the headline, cfg3 decode, cfg4 Zipf-skewed, cfg5 backward;
+                and the 128-expert layer of the decode shape at 512 .. 4096 tokens (between decode and prefill),
+                each against max(flop / MFMA peak, weight bytes / HBM peak)
   decode        the cfg3 entry again under the name the metric gives it
 """
 import argparse
@@ -95,7 +97,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle (no cpu_baseline, no parity)")
     ap.add_argument("--no-configs", action="store_true",
                     help="only the headline workload and its dominant kernel (for profiler runs)")
-    ap.add_argument("--only", default="", help="with --no-configs: also run this one of decode, zipf, readme, backward")
+    ap.add_argument("--only", default="", help="with --no-configs: also run this one of decode, mid, zipf, readme, backward")
     ap.add_argument("--extras", action="store_true",
                     help="also time the vendor library's dense GEMM on the two forward GEMM shapes, the routing and "
                          "permute kernels of the Zipf workload on their own, and the gate_up launch on zero weights "
@@ -170,7 +172,8 @@ def main():
             _cabi._p(d["hidden"]), _cabi._p(si), _cabi._p(d["gate_up_proj"]), _cabi._p(d["gate_up_proj_bias"]),
             _cabi._p(act), None, _cabi._p(sched), n_rows, K, E, H, I, _cabi.BF16, _cabi._stream())
     spin_up(gu_launch, args.spinup_ms / 2)
-    gu_ms = event_time_ms(gu_launch, args.steps)
+    kernel_iters = max(args.steps, 200)  # the isolated launches are timed over at least 200 of them whatever --steps says
+    gu_ms = event_time_ms(gu_launch, kernel_iters)
     y = _cabi.down(act, d["down_proj"], d["down_proj_bias"], sched)
 
     def dn_launch():
@@ -178,7 +181,7 @@ def main():
             _cabi._p(act), _cabi._p(d["down_proj"]), _cabi._p(d["down_proj_bias"]), _cabi._p(y), _cabi._p(sched),
             n_rows, E, H, I, _cabi.BF16, _cabi._stream())
     spin_up(dn_launch, args.spinup_ms / 2)
-    dn_ms = event_time_ms(dn_launch, args.steps)
+    dn_ms = event_time_ms(dn_launch, kernel_iters)
     gu_flop = n_rows * 4 * H * I
     gu_tflops = gu_flop / (gu_ms * 1e-3) / 1e12
     dn_tflops = n_rows * 2 * H * I / (dn_ms * 1e-3) / 1e12
@@ -186,7 +189,7 @@ def main():
     roofline = dict(bound="mfma", kernel="gemm_async_kernel<bf16, gate_up + clamped SwiGLU>", achieved=round(gu_tflops, 2),
                     peak=PEAK_BF16_TFLOPS, unit="TFLOP/s", frac=round(gu_tflops / PEAK_BF16_TFLOPS, 4),
                     traffic=traffic, traffic_source=traffic_source, algorithmic_flop_per_launch=gu_flop,
-                    avg_launch_ms=round(gu_ms, 4),
+                    avg_launch_ms=round(gu_ms, 4), launches_timed=kernel_iters,
                     down_gemm=dict(achieved=round(dn_tflops, 2), frac=round(dn_tflops / PEAK_BF16_TFLOPS, 4),
                                    avg_launch_ms=round(dn_ms, 4)))
     data_dependence = None
@@ -261,7 +264,7 @@ def main():
 
     # ---------------- cfg3: decode, 64 tokens, 128 experts ---------------------------------------------------
     decode = None
-    if wanted("decode"):
+    if wanted("decode") or wanted("mid"):
         dc = workloads.CONFIGS["decode"]
         Td, Ed, Kd = dc["T"], dc["E"], dc["K"]
         hostd, _ = workloads.make_config("decode", seed=0, weights=False)
@@ -304,6 +307,32 @@ def main():
                 b_ms = event_time_ms(bstep, args.steps)
                 decode_batches["tokens_%d" % tb] = dict(us=round(b_ms * 1e3, 1), active_experts=act_b,
                                                         gbs=round(nb / (b_ms * 1e-3) / 1e9, 1))
+        # ---------------- between decode and prefill: the same 128-expert layer at 512 .. 4096 tokens ----------
+        # (16 .. 128 rows per expert: every expert a single row tile; bound by the weight stream like the decode
+        # shape, with matrix work that grows with the tokens; reuses the decode workload's weights)
+        if wanted("mid"):
+            for name in ("mid512", "mid1024", "mid2048", "mid4096"):
+                mc = workloads.CONFIGS[name]
+                hostm, _ = workloads.make_config(name, seed=0, weights=False)
+                am = [hostm[k].to(dev) for k in ORDER[:3]] + ad[3:]
+                ms = timed(lambda: yamoe_amd.experts(*am, mc["T"], Ed, Kd), few)
+                cm = np.bincount(hostm["router_indices"].numpy().ravel(), minlength=Ed)
+                w_bytes = int((cm > 0).sum()) * 3 * H * I * 2
+                m_flop = mc["T"] * Kd * 6 * H * I
+                roof_ms = max(m_flop / (PEAK_BF16_TFLOPS * 1e12), w_bytes / (PEAK_HBM_GBS * 1e9)) * 1e3
+                entry = dict(ms=round(ms, 4), weight_gbs=round(w_bytes / (ms * 1e-3) / 1e9, 1),
+                             tflops=round(m_flop / (ms * 1e-3) / 1e12, 1), roofline_ms=round(roof_ms, 4),
+                             frac_of_roofline=round(roof_ms / ms, 4), rows_per_expert=[int(cm.min()), int(cm.max())],
+                             peak="max(flop / %.0f TFLOP/s, weight bytes / %.0f GB/s)" % (PEAK_BF16_TFLOPS, PEAK_HBM_GBS),
+                             parity=None)
+                if check and name in ("mid512", "mid4096"):
+                    got = yamoe_amd.experts(*am, mc["T"], Ed, Kd).float().cpu()
+                    want = O.experts_capacity(*([hostm[k] for k in ORDER[:3]] + [t.cpu() for t in ad[3:]]), mc["T"],
+                                              compute_dtype=torch.float32)
+                    entry["parity"] = parity_of(got, want, 1e-2, "fp32 oracle, all %d tokens, device-drawn weights copied back" % mc["T"])
+                    del got, want
+                configs["%s_128experts_forward_bf16" % name] = entry
+                del am
         del dd, ad
         torch.cuda.empty_cache()
 

@@ -125,7 +125,7 @@ def test_workloads_are_seeded_and_shaped():
     z, _ = make_config("zipf", seed=0, weights=False)
     counts = torch.bincount(z["router_indices"].flatten(), minlength=128)
     assert counts.max() > 10 * counts.float().mean() and (counts == 0).any()
-    assert set(CONFIGS) == {"readme", "gptoss20b", "decode", "zipf"}
+    assert set(CONFIGS) == {"readme", "gptoss20b", "decode", "zipf", "mid512", "mid1024", "mid2048", "mid4096"}
 
 
 def test_hub_layout_imports_as_yamoe(tmp_path):

@@ -54,7 +54,8 @@ def test_forward_and_backward_through_ctypes_with_reused_workspace(gpu, dtype):
                 r = O.route(d["router_indices"].numpy(), d["gate_up_proj"].shape[0], cap)
                 want_e, scale, _ = slot_terms(d, gy, oracle_act(d, r["sorted_idx"], 1), r["sorted_idx"], r["inv_pos"])
                 got_e = torch.gather(a.cpu().double(), 1, d["router_indices"])
-                assert torch.allclose(want_e, torch.gather(b.double(), 1, d["router_indices"]), rtol=1e-9, atol=1e-12)
+                b64 = O.experts_backward(gy, *[d[k] for k in KEYS], cap, compute_dtype=torch.float64)[1]
+                assert torch.allclose(want_e, torch.gather(b64, 1, d["router_indices"]), rtol=1e-9, atol=1e-12)
                 u = UNIT[dtype]
                 assert torch.all((got_e - want_e).abs() <= 2 * u * scale + 2 * u * want_e.abs() + 1e-30), (label, n)
                 continue

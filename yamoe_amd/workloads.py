@@ -9,6 +9,9 @@ same seed gives the same tensors on any machine) in fp32 and then cast.
   decode     64 tokens, E=128, top-4, bf16 (GPT-OSS-120B expert shape)
   zipf       16384 tokens, E=128, top-4, bf16, logits = randn + log Zipf(1.2) popularity
   (the backward workload is gptoss20b plus a randn grad_output)
+  mid512 .. mid4096  the 128-expert layer (GPT-OSS-120B expert shape) at 512, 1024, 2048 and 4096 tokens, top-4,
+             bf16: 16 to 128 rows per expert on average, between the decode and the prefill regime; every expert
+             is a single row tile and the layer is bound by the rate at which 6.4 GB of weights stream in
 """
 import math
 
@@ -24,6 +27,9 @@ CONFIGS = {
     "zipf": dict(T=16384, H=2880, I=2880, E=128, K=4, dtype=torch.bfloat16, w_std=0.02, bias_std=0.02, renorm=True,
                  zipf=1.2),
 }
+for _t in (512, 1024, 2048, 4096):
+    CONFIGS["mid%d" % _t] = dict(T=_t, H=2880, I=2880, E=128, K=4, dtype=torch.bfloat16, w_std=0.02, bias_std=0.02,
+                                 renorm=True, zipf=0.0)
 
 
 def make_routing(T, E, K, gen, renorm=True, zipf=0.0):
