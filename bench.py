@@ -24,6 +24,7 @@ Also on the line:
   decode        the cfg3 entry again under the name the metric gives it
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -100,8 +101,9 @@ def main():
     ap.add_argument("--only", default="", help="with --no-configs: also run this one of decode, mid, zipf, readme, backward")
     ap.add_argument("--extras", action="store_true",
                     help="also time the vendor library's dense GEMM on the two forward GEMM shapes, the routing and "
-                         "permute kernels of the Zipf workload on their own, and the gate_up launch on zero weights "
-                         "(how much of its time is the power limit)")
+                         "permute kernels of the Zipf workload on their own, the gate_up launch on zero weights "
+                         "(how much of its time is the power limit) and a register-only MFMA loop on random and on "
+                         "zero operands (what the matrix pipes sustain with nothing else going on)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy kernel (a known FETCH_SIZE / WRITE_SIZE for counter runs)")
     args = ap.parse_args()
@@ -395,6 +397,24 @@ def main():
         torch.cuda.empty_cache()
 
     if args.extras:
+        # What the matrix pipes themselves sustain: a register-only loop of v_mfma_f32_32x32x16_bf16 (one wave per SIMD
+        # on every CU, 4 x 4 accumulator blocks: the forward tile's wave shape, no memory traffic) on pseudo-random and
+        # on all-zero operands.  The part runs against its power limit, so the two differ; the random-operand figure,
+        # not the 2.5 PFLOP/s peak, is the ceiling of any bf16 GEMM on real data here.
+        sink = torch.zeros(4, device=dev)
+        flop_out = ctypes.c_double(0.0)
+        cus = torch.cuda.get_device_properties(dev).multi_processor_count
+        probe = {}
+        for label, rnd in (("random_operands", 1), ("zero_operands", 0)):
+            def mfma_loop():
+                rc = _cabi.lib().yamoe_probe_mfma_rate(cus, 4000, rnd, _cabi._p(sink), ctypes.byref(flop_out), _cabi._stream())
+                assert rc == 0
+            spin_up(mfma_loop, args.spinup_ms)
+            ms = event_time_ms(mfma_loop, 20)
+            probe[label] = dict(ms=round(ms, 4), tflops=round(flop_out.value / (ms * 1e-3) / 1e12, 1),
+                                frac_of_peak=round(flop_out.value / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4))
+        probe["workgroups"] = cus
+        extras["mfma_register_loop"] = probe
         # For scale: the vendor library's dense GEMM (torch.matmul) on the same flop counts and operand layouts as the
         # two forward GEMMs: [T*K, H] x [H, 2I] and [T*K, I] x [I, H], one matrix instead of 32 experts, no bias, no GLU.
         gl = torch.Generator(device=dev).manual_seed(7)

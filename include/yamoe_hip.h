@@ -24,7 +24,8 @@ extern "C" {
 #endif
 
 /* 2: YAMOE_F64 dtype code; yamoe_experts_forward_static; yamoe_route_workspace_bytes returns the size of a
- *    segments x buckets table above 4096 assignments (it was a constant 256 bytes); stream_max_rows up to 32. */
+ *    segments x buckets table above 4096 assignments (it was a constant 256 bytes); stream_max_rows up to 32;
+ *    yamoe_probe_mfma_rate. */
 #define YAMOE_ABI_VERSION 2
 
 /* element type of activations, weights, biases and routing weights.  YAMOE_F64 is taken by the row movers among
@@ -219,6 +220,16 @@ int yamoe_batch_mm(const void *x, const void *weights, void *output, int32_t E, 
 int yamoe_router_topk(const void *hidden, const void *weight, const void *bias, int32_t T, int32_t H,
                       int32_t E, int32_t top_k, int32_t dtype, int64_t *router_indices,
                       void *router_scores, void *topk_weights, void *logits, void *stream);
+
+/* ---- diagnostics ---------------------------------------------------------------------------
+ * No counterpart in the reference; not on the path of any op.  A register-only loop of
+ * v_mfma_f32_32x32x16_bf16 (one wave per SIMD in each of `workgroups` workgroups of 256 threads,
+ * 4 x 4 accumulator blocks, `iters` rounds of 16 MFMAs, no memory traffic in the loop) on
+ * pseudo-random (random_operands != 0) or all-zero operands: the rate the matrix pipes of this
+ * part sustain, for scale next to the expert GEMMs (the part runs against its power limit, so
+ * the rate depends on the operand values).  *flop receives the flop count of the launch. */
+int yamoe_probe_mfma_rate(int32_t workgroups, int32_t iters, int32_t random_operands, float *sink,
+                          double *flop, void *stream);
 
 #ifdef __cplusplus
 }

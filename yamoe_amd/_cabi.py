@@ -24,7 +24,7 @@ SYMBOLS = [
     "yamoe_experts_backward_workspace_bytes",
     "yamoe_experts_backward", "yamoe_sort_workspace_bytes", "yamoe_sort", "yamoe_bincount_cumsum", "yamoe_padded_gather",
     "yamoe_padded_scatter_workspace_bytes", "yamoe_padded_scatter", "yamoe_index_select", "yamoe_regular_groups",
-    "yamoe_batch_mm_workspace_bytes", "yamoe_batch_mm", "yamoe_router_topk",
+    "yamoe_batch_mm_workspace_bytes", "yamoe_batch_mm", "yamoe_router_topk", "yamoe_probe_mfma_rate",
 ]
 
 
@@ -66,6 +66,7 @@ def lib():
         L.yamoe_experts_backward_workspace_bytes.argtypes = [pp]
         L.yamoe_experts_backward.argtypes = [pp] + [vp] * 15 + [sz, vp]
         L.yamoe_router_topk.argtypes = [vp, vp, vp, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp]
+        L.yamoe_probe_mfma_rate.argtypes = [i32, i32, i32, vp, ctypes.POINTER(ctypes.c_double), vp]
         _lib = L
     return _lib
 

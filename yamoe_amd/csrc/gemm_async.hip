@@ -76,7 +76,21 @@ struct Args {
   // row times dot_with[row][same columns] (a [rows, ldc] tensor), summed over the wave's 128 columns
   const void *dot_with;
   float *dot_part;
+#ifdef YAMOE_TILE_STAMPS
+  unsigned long long *stamps;  // [stamps_cap][8]: see yamoe_debug_tile_stamps
+  int stamps_cap;
+#endif
 };
+
+#ifdef YAMOE_TILE_STAMPS
+// Diagnostic build (-DYAMOE_TILE_STAMPS, `python -m yamoe_amd.tile_stamps`): thread 0 of every tile of gemm_async_kernel
+// leaves eight words at stamps[8 * flat tile index]: the shader clock (s_memtime) at workgroup entry, before the first
+// copy, when the first slab has landed, after the contraction loop, before the row-wise stores and at the end, then
+// valid rows | valid columns << 16, and where it ran (XCC id << 8 | SE, SH and CU id).
+#define YAMOE_STAMP(i) if (tid == 0) stamp_reg[i] = __builtin_amdgcn_s_memtime()
+#else
+#define YAMOE_STAMP(i)
+#endif
 
 template <typename T> struct Mma;
 template <> struct Mma<bf16_t> {
@@ -124,6 +138,10 @@ template <bool P1A_, bool P1B_, bool P2A_, bool P2B_, bool NEXT_, int VM_, bool 
 
 struct TileInfo {
   int expert, row0, rows_valid, n0;
+#ifdef YAMOE_TILE_STAMPS
+  int slot;
+  unsigned long long t_entry, t_lookup;
+#endif
 };
 
 // NMI / NNI: how many of this wave's four 32-row and four 32-column blocks of the tile hold valid rows / columns.  The
@@ -132,7 +150,7 @@ struct TileInfo {
 // MFMAs instead of all of them to one.
 // NAB: how many of the tile's eight 32-row blocks are copied (the others hold no valid row).
 template <typename T, int EPI, int NMI, bool BNK, int NNI = 4, int NAB = 8>
-__device__ inline void run_tile(const Args &args, const TileInfo &ti, const int tid, const char *a_base,
+__device__ __forceinline__ void run_tile(const Args &args, const TileInfo &ti, const int tid, const char *a_base,
                                 const uint32_t (&a_off)[8], const char *b_base, const uint32_t (&b_off)[8],
                                 long long b_slab_bytes) {
   const int lane = tid & 63;
@@ -151,6 +169,9 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
       for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
 
   const int n_slabs = args.Kd / kBK;  // even: the contraction length is a multiple of 64
+#ifdef YAMOE_TILE_STAMPS
+  unsigned long long stamp_reg[6] = {ti.t_entry, ti.t_lookup, 0, 0, 0, 0};
+#endif
 
   // The tile's bias values, one per thread, requested before anything else: they are the oldest entry of the memory
   // queue, so the first wait of the pipeline covers them, and the epilogue finds them in a register instead of
@@ -292,6 +313,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
   __syncthreads();
+  YAMOE_STAMP(2);
   read_frags(0, 0, fa0, fb0);
 
   // The instruction order is fixed by hand, because one wave per SIMD has nobody to hide behind: every LDS
@@ -394,6 +416,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
     }
   }
 
+  YAMOE_STAMP(3);
   // ---- epilogue -------------------------------------------------------------------------------------
   // The output tile is staged in LDS (the slab ring is dead by now) as [row][column] and then written
   // out row by row with 16 bytes per lane, so that a wave stores whole 512-byte (or 256-byte) row
@@ -506,6 +529,7 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
   if constexpr (EPI == EPI_STORE) {
     stage_biased(std::false_type());
     __syncthreads();
+    YAMOE_STAMP(4);
     store_rows((T *)args.C, args.ldc, n0, kBN, args.Nd);
   } else {
     if (args.C2 != nullptr) {  // pre-activations for the backward: the biased product itself
@@ -532,8 +556,21 @@ __device__ inline void run_tile(const Args &args, const TileInfo &ti, const int 
         }
     }
     __syncthreads();
+    YAMOE_STAMP(4);
     store_rows((T *)args.C, args.ldc, n0 >> 1, kBN / 2, args.Nd >> 1);
   }
+#ifdef YAMOE_TILE_STAMPS
+  YAMOE_STAMP(5);
+  if (tid == 0 && args.stamps != nullptr && ti.slot < args.stamps_cap) {
+    unsigned long long *o = args.stamps + 8ll * ti.slot;
+#pragma unroll
+    for (int i = 0; i < 6; ++i) o[i] = stamp_reg[i];
+    o[6] = (unsigned long long)(uint32_t)ti.rows_valid | ((unsigned long long)(uint32_t)min(kBN, args.Nd - ti.n0) << 16);
+    const unsigned hw = __builtin_amdgcn_s_getreg((4 << 0) | (8 << 6) | (7 << 11));    // HW_ID bits 8..15: CU, SH and SE id
+    const unsigned xcc = __builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (3 << 11));  // XCC_ID
+    o[7] = ((unsigned long long)xcc << 8) | hw;
+  }
+#endif
 }
 
 template <typename T, int EPI, bool GATHER, bool BNK>
@@ -544,6 +581,9 @@ __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
   // the same weight slabs meet in one L2.  A share longer than gridDim.x / 8 hands its excess to the workgroups
   // of shorter shares (the grid has at least as many workgroups as there are tiles).
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1;
+#ifdef YAMOE_TILE_STAMPS
+  const unsigned long long t_entry = __builtin_amdgcn_s_memtime();
+#endif
   int L;
   {
     const int xcd = blockIdx.x % kXcds, i = blockIdx.x / kXcds, slots = gridDim.x / kXcds;
@@ -575,13 +615,21 @@ __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
   {
     const int *tiles = args.sched + kSchedHeader;
     int t0 = fast_div(L, args.n_col_div);
-    int gfirst = tiles[8 * t0 + 3], gcount = tiles[8 * t0 + 4];
-    FastDiv by_gcount = {(uint32_t)tiles[8 * t0 + 5], (uint32_t)tiles[8 * t0 + 6]};
+    int gfirst = __builtin_amdgcn_readfirstlane(tiles[8 * t0 + 3]), gcount = __builtin_amdgcn_readfirstlane(tiles[8 * t0 + 4]);
+    FastDiv by_gcount = {(uint32_t)__builtin_amdgcn_readfirstlane(tiles[8 * t0 + 5]),
+                         (uint32_t)__builtin_amdgcn_readfirstlane(tiles[8 * t0 + 6])};
     int local = L - gfirst * args.n_col_tiles;
     int col_tile = fast_div(local, by_gcount);
     const int *te = tiles + 8 * (gfirst + local - col_tile * gcount);
-    ti.expert = te[0]; ti.row0 = te[1]; ti.rows_valid = te[2];
+    // (the same for every lane; said explicitly, so that the operand addresses built from them stay in scalar registers
+    // whatever the compiler can prove about the work list's memory)
+    ti.expert = __builtin_amdgcn_readfirstlane(te[0]);
+    ti.row0 = __builtin_amdgcn_readfirstlane(te[1]);
+    ti.rows_valid = __builtin_amdgcn_readfirstlane(te[2]);
     ti.n0 = col_tile * kBN;
+#ifdef YAMOE_TILE_STAMPS
+    ti.slot = L; ti.t_entry = t_entry;
+#endif
   }
 
   // A copies: copy i fetches rows 32*i + 8*wave + (lane >> 3); LDS position lane & 7 holds piece pos ^ ((row >> 1) & 7)
@@ -629,6 +677,11 @@ __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
     b_slab_bytes = kBK * b_ld_bytes;
   }
 
+#ifdef YAMOE_TILE_STAMPS
+  // (after the work-list look-ups and the gathered row numbers: a_off depends on both)
+  asm volatile("s_waitcnt vmcnt(0)" : : "v"(a_off[0]), "v"(a_off[7]) : "memory");
+  ti.t_lookup = __builtin_amdgcn_s_memtime();
+#endif
   const int n_blocks32 = (ti.rows_valid + 31) >> 5;
   const int n_mi = (n_blocks32 - wm + 1) >> 1;
   // valid 32-column blocks of this wave column (they alternate between the two); tiles of 64 or 128 valid columns with
@@ -658,6 +711,11 @@ __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
 #undef YAMOE_RUN6
 }
 
+#ifdef YAMOE_TILE_STAMPS
+static unsigned long long *g_tile_stamps = nullptr;
+static int g_tile_stamps_cap = 0;
+#endif
+
 template <typename T, int EPI, bool GATHER, bool BNK>
 static int launch(const Args &args, int max_row_tiles, hipStream_t stream) {
   auto kernel = gemm_async_kernel<T, EPI, GATHER, BNK>;
@@ -667,7 +725,14 @@ static int launch(const Args &args, int max_row_tiles, hipStream_t stream) {
   long long total = (long long)max_row_tiles * args.n_col_tiles;
   if (total <= 0) return 0;
   total = (total + kXcds - 1) / kXcds * kXcds;
+#ifdef YAMOE_TILE_STAMPS
+  Args stamped = args;
+  stamped.stamps = g_tile_stamps;
+  stamped.stamps_cap = g_tile_stamps_cap;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(kThreads), lds_bytes, stream, stamped);
+#else
   hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(kThreads), lds_bytes, stream, args);
+#endif
   return check_launch("gemm_async_kernel");
 }
 
@@ -1076,6 +1141,15 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_small_kernel(const WgradArg
 }
 
 }  // namespace async
+
+#ifdef YAMOE_TILE_STAMPS
+// Where the next launches of gemm_async_kernel leave their per-tile clock stamps (device memory, 8 words per tile, room
+// for `tiles` tiles; nullptr switches them off).  Exported by the diagnostic build only.
+extern "C" void yamoe_debug_tile_stamps(void *buffer, int32_t tiles) {
+  async::g_tile_stamps = (unsigned long long *)buffer;
+  async::g_tile_stamps_cap = buffer ? tiles : 0;
+}
+#endif
 
 // True when the asynchronous-copy kernels can take this product.
 bool gemm_async_supported(int Kd, int Nd, int lda, int ldb, long long a_span_bytes) {
