@@ -25,7 +25,7 @@ extern "C" {
 
 /* 2: YAMOE_F64 dtype code; yamoe_experts_forward_static; yamoe_route_workspace_bytes returns the size of a
  *    segments x buckets table above 4096 assignments (it was a constant 256 bytes); stream_max_rows up to 32;
- *    yamoe_probe_mfma_rate. */
+ *    yamoe_probe_mfma_rate; yamoe_router_topk takes fp32; yamoe_router_backward. */
 #define YAMOE_ABI_VERSION 2
 
 /* element type of activations, weights, biases and routing weights.  YAMOE_F64 is taken by the row movers among
@@ -211,15 +211,28 @@ int yamoe_batch_mm(const void *x, const void *weights, void *output, int32_t E, 
                    void *stream);
 
 /* The router step of Yamoe.forward (torch-ext/yamoe/layers.py:128-152; GptOssTopKRouter.forward,
- * torch-ext/yamoe/vendored/gpt_oss_mlp.py:128-142) in one kernel, 16-bit dtypes:
+ * torch-ext/yamoe/vendored/gpt_oss_mlp.py:128-142) in one kernel:
  *   logits = round(hidden . weight^T + bias)            [T,E]  (optional output)
  *   router_indices = top_k experts by logit, descending; equal logits: lower expert id first   [T,K] int64
  *   router_scores  = softmax over the K picked logits (fp32, rounded once), scattered into a
  *                    zero [T,E] row; topk_weights (optional) holds the same K values as [T,K].
- * H must be a multiple of 16, E <= 256, top_k <= min(E, 16).  bias may be NULL. */
+ * H must be a multiple of 16 (fp32: of 8), E <= 256, top_k <= min(E, 16).  bias may be NULL.  All three dtypes. */
 int yamoe_router_topk(const void *hidden, const void *weight, const void *bias, int32_t T, int32_t H,
                       int32_t E, int32_t top_k, int32_t dtype, int64_t *router_indices,
                       void *router_scores, void *topk_weights, void *logits, void *stream);
+
+/* The gradient of that step (what autograd gives through the reference's four torch calls, layers.py:128-149):
+ * from d_scores [T,E], the gradient of the dense router_scores, with p_k = router_scores[t, e_k] and
+ * g_k = d_scores[t, e_k] at the token's picks e_k:
+ *   d_logits[t, e_k] = p_k (g_k - sum_j p_j g_j), zero at every other expert
+ *   d_hidden [T,H] = d_logits . weight     (the router's share of the hidden-state gradient; add the experts' share)
+ *   d_weight [E,H] = d_logits^T . hidden,  d_bias [E] = column sums of d_logits  (d_bias may be NULL)
+ * All tensors in the activation dtype, fp32 accumulation.  H and E multiples of 8 (fp32: of 4). */
+size_t yamoe_router_backward_workspace_bytes(int32_t T, int32_t E, int32_t dtype);
+int yamoe_router_backward(const void *d_scores, const int64_t *router_indices, const void *router_scores,
+                          const void *hidden, const void *weight, int32_t T, int32_t H, int32_t E,
+                          int32_t top_k, int32_t dtype, void *d_hidden, void *d_weight, void *d_bias,
+                          void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- diagnostics ---------------------------------------------------------------------------
  * No counterpart in the reference; not on the path of any op.  A register-only loop of

@@ -18,7 +18,7 @@ def draw(T, H, E, dtype, seed, bias=True):
     return x, w, b
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("T,H,E,K", [(4096, 2880, 32, 4), (64, 2880, 128, 4), (1, 64, 8, 2), (77, 128, 5, 5), (300, 256, 200, 16),
                                      (33, 48, 33, 1)])
 def test_router_topk(gpu, dtype, T, H, E, K):
@@ -30,15 +30,22 @@ def test_router_topk(gpu, dtype, T, H, E, K):
     idx, scores, topw, logits = idx.cpu(), scores.cpu(), topw.cpu(), logits.cpu()
     # the linear: fp32 accumulation in another order than the oracle's, so a logit may land one rounding step away
     _, _, want_logits = O.router(x, w, b, K)
-    ulp = 2.0 ** (-7 if dtype == torch.bfloat16 else -10)
-    diff = (logits.float() - want_logits.float()).abs()
-    assert torch.all(diff <= ulp * torch.maximum(want_logits.float().abs(), torch.full_like(diff, 2.0 ** -6)) + 1e-6)
-    assert (diff > 0).float().mean() < 0.05
+    ulp = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10, torch.float32: 2.0 ** -18}[dtype]
+    if dtype == torch.float32:
+        # nothing is rounded but the fp32 accumulation itself: against the fp64 product, within 2^-20 of the sum of the
+        # terms' magnitudes
+        want64 = x.double() @ w.double().t() + (b.double() if b is not None else 0.0)
+        scale = x.double().abs() @ w.double().abs().t() + (b.double().abs() if b is not None else 0.0)
+        assert torch.all((logits.double() - want64).abs() <= 2.0 ** -20 * scale + 1e-30)
+    else:
+        diff = (logits.float() - want_logits.float()).abs()
+        assert torch.all(diff <= ulp * torch.maximum(want_logits.float().abs(), torch.full_like(diff, 2.0 ** -6)) + 1e-6)
+        assert (diff > 0).float().mean() < 0.05
     # top-k, softmax and scatter on the kernel's own logits: picks bit-exact (ties included), weights within one rounding step
     want_idx, want_scores = O.router_from_logits(logits, K)
     assert torch.equal(idx, want_idx)
     assert torch.all((scores.float() - want_scores.float()).abs() <= ulp * want_scores.float())
-    assert (scores != want_scores).float().mean() < 0.01
+    assert dtype == torch.float32 or (scores != want_scores).float().mean() < 0.01   # (fp32: the last bit of expf)
     assert torch.equal(torch.gather(scores, 1, idx), topw)
     assert torch.equal(scores != 0, torch.zeros_like(scores, dtype=torch.bool).scatter_(1, idx, topw != 0))
 
@@ -60,7 +67,7 @@ def test_router_rejects(gpu):
     import yamoe_amd
     x, w, b = draw(8, 64, 4, torch.bfloat16, 0)
     with pytest.raises(RuntimeError):
-        yamoe_amd.router_topk(x.float().to(gpu), w.float().to(gpu), b.float().to(gpu), 2)      # fp32: not taken
+        yamoe_amd.router_topk(x.double().to(gpu), w.double().to(gpu), b.double().to(gpu), 2)   # fp64: not taken
     with pytest.raises(RuntimeError):
         yamoe_amd.router_topk(x.to(gpu), w.to(gpu), b.to(gpu), 5)                               # top_k > E
     with pytest.raises(RuntimeError):
@@ -184,3 +191,30 @@ def test_yamoe_layer_trains_the_router(gpu, dtype):
     for n, a, b in zip(names, got, want):
         assert a is not None, n
         assert report("router training " + n, a.cpu().double(), b.double(), tol) < tol, n
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,H,E,K", [(4096, 2880, 32, 4), (300, 256, 128, 4), (5, 64, 8, 2), (1000, 320, 40, 3), (20, 64, 16, 16)])
+def test_router_backward(gpu, dtype, T, H, E, K):
+    """yamoe_router_backward against autograd through the oracle's router step on the kernel's own picks: gradients of
+    hidden states, router weight and router bias from a random gradient of the dense scores (torch-ext/yamoe/layers.py:
+    128-149 differentiated)."""
+    from yamoe_amd import _cabi
+    print("router backward", dtype, T, H, E, K, flush=True)
+    x, w, b = draw(T, H, E, dtype, 3 * T + E)
+    idx, scores, _, _ = _cabi.router_topk(x.to(gpu), w.to(gpu), b.to(gpu), K)
+    g = torch.randn(T, E, generator=torch.Generator().manual_seed(T)).to(dtype)
+    d_x, d_w, d_b = _cabi.router_backward(g.to(gpu), idx, scores, x.to(gpu), w.to(gpu), K)
+    torch.cuda.synchronize()
+    cd = torch.float64 if dtype == torch.float32 else torch.float32
+    leaves = [t.to(cd).requires_grad_(True) for t in (x, w, b)]
+    _, want_scores, _ = O.router(*leaves, K, compute_dtype=cd, picks=idx.cpu())
+    want = torch.autograd.grad(want_scores, leaves, g.to(cd))
+    tol = 1e-5 if dtype == torch.float32 else 2e-2   # 16-bit: d_logits and the stored scores are rounded on the way
+    for name, got, ref in zip(("d_hidden", "d_weight", "d_bias"), (d_x, d_w, d_b), want):
+        assert report("router backward " + name, got.cpu().double(), ref.double(), tol) < tol, name
+    # only the picked experts carry a gradient: with d_scores zero at the picks everything vanishes
+    g0 = g.clone().scatter_(1, idx.cpu(), 0.0)
+    z_x, z_w, z_b = _cabi.router_backward(g0.to(gpu), idx, scores, x.to(gpu), w.to(gpu), K)
+    torch.cuda.synchronize()
+    assert float(z_x.abs().max()) == 0 and float(z_w.abs().max()) == 0 and float(z_b.abs().max()) == 0

@@ -5,7 +5,7 @@ Same surface as the reference package for this path (torch-ext/yamoe/__init__.py
 the C ABI of libyamoe_hip.so; the first use of any of them fails if the native libraries are not built.
 """
 _OPS = ("gather", "scatter", "sort", "bincount_cumsum", "index_select_out", "batch_mm", "experts", "experts_backward",
-        "router_topk")
+        "router_topk", "router_topk_backward")
 _LAYERS = ("Yamoe", "experts_autograd")
 
 __all__ = ["ops", *_LAYERS, *_OPS]

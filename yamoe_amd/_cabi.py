@@ -25,6 +25,7 @@ SYMBOLS = [
     "yamoe_experts_backward", "yamoe_sort_workspace_bytes", "yamoe_sort", "yamoe_bincount_cumsum", "yamoe_padded_gather",
     "yamoe_padded_scatter_workspace_bytes", "yamoe_padded_scatter", "yamoe_index_select", "yamoe_regular_groups",
     "yamoe_batch_mm_workspace_bytes", "yamoe_batch_mm", "yamoe_router_topk", "yamoe_probe_mfma_rate",
+    "yamoe_router_backward_workspace_bytes", "yamoe_router_backward",
 ]
 
 
@@ -66,6 +67,9 @@ def lib():
         L.yamoe_experts_backward_workspace_bytes.argtypes = [pp]
         L.yamoe_experts_backward.argtypes = [pp] + [vp] * 15 + [sz, vp]
         L.yamoe_router_topk.argtypes = [vp, vp, vp, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp]
+        L.yamoe_router_backward_workspace_bytes.restype = sz
+        L.yamoe_router_backward_workspace_bytes.argtypes = [i32, i32, i32]
+        L.yamoe_router_backward.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp, vp, vp, vp, sz, vp]
         L.yamoe_probe_mfma_rate.argtypes = [i32, i32, i32, vp, ctypes.POINTER(ctypes.c_double), vp]
         _lib = L
     return _lib
@@ -180,6 +184,23 @@ def router_topk(hidden, weight, bias, top_k):
     _check(lib().yamoe_router_topk(_p(hidden), _p(weight), _p(bias), T, H, E, top_k, dtype_code(hidden), _p(idx), _p(scores),
                                    _p(topw), _p(logits), _stream()), "yamoe_router_topk")
     return idx, scores, topw, logits
+
+
+def router_backward(d_scores, router_indices, router_scores, hidden, weight, top_k, want_bias=True):
+    """yamoe_router_backward: (d_hidden [T,H], d_weight [E,H], d_bias [E] or None)."""
+    _need_gpu(d_scores, router_indices, router_scores, hidden, weight)
+    T, H = hidden.shape
+    E = weight.shape[0]
+    d_hidden = torch.empty_like(hidden)
+    d_weight = torch.empty_like(weight)
+    d_bias = torch.empty(E, dtype=hidden.dtype, device=hidden.device) if want_bias else None
+    need = lib().yamoe_router_backward_workspace_bytes(T, E, dtype_code(hidden))
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=hidden.device)
+    _check(lib().yamoe_router_backward(_p(d_scores.contiguous()), _p(router_indices.contiguous()), _p(router_scores.contiguous()),
+                                       _p(hidden.contiguous()), _p(weight.contiguous()), T, H, E, top_k, dtype_code(hidden),
+                                       _p(d_hidden), _p(d_weight), _p(d_bias), _p(ws), need, _stream()),
+           "yamoe_router_backward")
+    return d_hidden, d_weight, d_bias
 
 
 def problem(hidden, router_indices, routing_weights, gate_up_proj, capacity):

@@ -21,7 +21,7 @@ for _p in (_LIB_HIP, _LIB_OPS):
 torch.ops.load_library(_LIB_OPS)
 ops = torch.ops._yamoe_amd_ops
 for _name in ("experts", "experts_backward", "gather", "scatter", "sort", "bincount_cumsum", "index_select_out", "batch_mm",
-              "router_topk"):
+              "router_topk", "router_topk_backward"):
     if not hasattr(ops, _name):
         raise ImportError("%s is stale (no operator %r): rebuild with `python -m yamoe_amd.build`" % (_LIB_OPS, _name))
 

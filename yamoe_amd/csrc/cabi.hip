@@ -95,6 +95,9 @@ int gemm_f32_gate_up(const void *, const int *, const void *, const void *, void
 int gemm_f32_down(const void *, const void *, const void *, void *, const void *, int, int, int, int, hipStream_t);
 bool wgrad_async_supported(int Md, int Nd);
 
+template <typename T>
+int launch_router_backward_logits(const void *, const long long *, const void *, int, int, int, void *, hipStream_t);
+
 template <typename T> struct HasStreamPath { static constexpr bool value = sizeof(T) == 2; };
 
 // The MFMA tile kernels for the two forward products: the asynchronous-copy pipeline when the dtype
@@ -545,6 +548,75 @@ extern "C" int yamoe_experts_backward(const yamoe_problem *p, const void *grad_o
                                             gate_up_proj_bias, down_proj, down_proj_bias, d_hidden, d_routing,
                                             d_gate_up_proj, d_gate_up_proj_bias, d_down_proj, d_down_proj_bias,
                                             workspace, (hipStream_t)stream));
+}
+
+// ---- gradient of the router step ------------------------------------------------------------------------
+// d_logits from the softmax over the picks (router.hip), then the two products and the column sums on the expert
+// layer's own kernels, with the whole batch as the one "expert": d_hidden = d_logits . W (a [T, E] x [E, H] product of
+// rows), d_weight = d_logits^T . hidden (a weight-gradient product over the T rows), d_bias = column sums.
+struct RouterBackwardBuffers {
+  void *d_logits, *schedule;
+  int *counts, *offsets;
+  size_t schedule_bytes;
+};
+static size_t carve_router_backward(int T, int E, int dtype, void *ws, RouterBackwardBuffers *b) {
+  Carver c(ws);
+  b->d_logits = c.take((size_t)T * E * dtype_size(dtype));
+  b->counts = (int *)c.take(4);
+  b->offsets = (int *)c.take(8);
+  b->schedule_bytes = yamoe_schedule_bytes(T, 1);
+  b->schedule = c.take(b->schedule_bytes);
+  return c.used;
+}
+
+extern "C" size_t yamoe_router_backward_workspace_bytes(int32_t T, int32_t E, int32_t dtype) {
+  if (T < 0 || E <= 0 || (dtype != YAMOE_F32 && dtype != YAMOE_F16 && dtype != YAMOE_BF16)) return 0;
+  RouterBackwardBuffers b;
+  return carve_router_backward(T, E, dtype, nullptr, &b);
+}
+
+template <typename T>
+static int router_backward_impl(const void *d_scores, const long long *indices, const void *scores, const void *hidden,
+                                const void *weight, int Tn, int H, int E, int K, void *d_hidden, void *d_weight,
+                                void *d_bias, void *ws, hipStream_t stream) {
+  RouterBackwardBuffers b;
+  carve_router_backward(Tn, E, ElemTraits<T>::kDtype, ws, &b);
+  YAMOE_TRY(launch_router_backward_logits<T>(d_scores, indices, scores, Tn, E, K, b.d_logits, stream));
+  YAMOE_TRY(yamoe_regular_groups(b.counts, b.offsets, 1, Tn, (void *)stream));
+  const int stream_rows = HasStreamPath<T>::value ? kStreamMaxRows : 0;
+  YAMOE_TRY(yamoe_build_schedule(b.counts, b.offsets, Tn, 1, Tn, stream_rows, b.schedule, b.schedule_bytes, (void *)stream));
+  // d_hidden [T, H] = d_logits [T, E] . weight [E, H]: the down-projection launchers compute rows[., Kd] x w[Kd, Nd]
+  YAMOE_TRY(down_both<T>(b.d_logits, weight, nullptr, d_hidden, b.schedule, Tn, 1, /*H=*/H, /*I=*/E, stream));
+  // d_weight [E, H] = d_logits^T . hidden, contraction over the T rows (the register-staged kernel: it reads nothing
+  // past the end of the caller's tensors)
+  YAMOE_TRY(gemm_wgrad<T>(b.d_logits, hidden, d_weight, b.counts, b.offsets, Tn, 1, /*Md=*/E, /*Nd=*/H, stream));
+  if (d_bias != nullptr) YAMOE_TRY(launch_expert_colsum<T>(b.d_logits, b.counts, b.offsets, Tn, d_bias, 1, E, stream));
+  return 0;
+}
+
+extern "C" int yamoe_router_backward(const void *d_scores, const int64_t *router_indices, const void *router_scores,
+                                     const void *hidden, const void *weight, int32_t T_, int32_t H, int32_t E,
+                                     int32_t top_k, int32_t dtype, void *d_hidden, void *d_weight, void *d_bias,
+                                     void *workspace, size_t workspace_bytes, void *stream) {
+  YAMOE_TRY(check_gemm_shape("yamoe_router_backward", T_, 1, H, E, dtype));
+  if (top_k <= 0 || top_k > E) { set_error("yamoe_router_backward: need 1 <= top_k <= E"); return YAMOE_E_ARG; }
+  if (!d_weight) { set_error("yamoe_router_backward: null pointer"); return YAMOE_E_ARG; }
+  if (T_ == 0) {
+    YAMOE_TRY(fill_zero(d_weight, (size_t)E * H * dtype_size(dtype), (hipStream_t)stream));
+    if (d_bias) YAMOE_TRY(fill_zero(d_bias, (size_t)E * dtype_size(dtype), (hipStream_t)stream));
+    return 0;
+  }
+  if (!d_scores || !router_indices || !router_scores || !hidden || !weight || !d_hidden || !workspace) {
+    set_error("yamoe_router_backward: null pointer");
+    return YAMOE_E_ARG;
+  }
+  if (workspace_bytes < yamoe_router_backward_workspace_bytes(T_, E, dtype)) {
+    set_error("yamoe_router_backward: workspace too small");
+    return YAMOE_E_WORKSPACE;
+  }
+  YAMOE_DISPATCH(dtype, router_backward_impl<T>(d_scores, (const long long *)router_indices, router_scores, hidden, weight,
+                                                T_, H, E, top_k, d_hidden, d_weight, d_bias, workspace,
+                                                (hipStream_t)stream));
 }
 
 // ---- batch_mm on the regular [E, C, *] layout -------------------------------------------------------

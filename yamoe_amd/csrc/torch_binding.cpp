@@ -284,8 +284,6 @@ std::tuple<at::Tensor, at::Tensor> router_topk_op(const at::Tensor &hidden, cons
   TORCH_CHECK(hidden.is_cuda() && weight.is_cuda(), "router_topk: GPU tensors only");
   TORCH_CHECK(hidden.dim() == 2 && weight.dim() == 2 && hidden.size(1) == weight.size(1),
               "router_topk: hidden [T, H] and weight [E, H] expected");
-  TORCH_CHECK(hidden.scalar_type() == at::kBFloat16 || hidden.scalar_type() == at::kHalf,
-              "router_topk: bf16 or fp16 activations only");
   TORCH_CHECK(weight.scalar_type() == hidden.scalar_type(), "router_topk: weight dtype must match hidden");
   const int64_t T = hidden.size(0), H = hidden.size(1), E = weight.size(0);
   at::Tensor x = hidden.contiguous(), w = weight.contiguous(), b;
@@ -305,11 +303,43 @@ std::tuple<at::Tensor, at::Tensor> router_topk_op(const at::Tensor &hidden, cons
   return std::make_tuple(indices, scores);
 }
 
+// gradient of router_topk with respect to hidden, weight and bias, from the gradient of the dense scores
+std::tuple<at::Tensor, at::Tensor, at::Tensor> router_topk_backward_op(const at::Tensor &d_scores, const at::Tensor &indices,
+                                                                       const at::Tensor &scores, const at::Tensor &hidden,
+                                                                       const at::Tensor &weight) {
+  TORCH_CHECK(d_scores.is_cuda() && indices.is_cuda() && scores.is_cuda() && hidden.is_cuda() && weight.is_cuda(),
+              "router_topk_backward: GPU tensors only");
+  TORCH_CHECK(hidden.dim() == 2 && weight.dim() == 2 && hidden.size(1) == weight.size(1),
+              "router_topk_backward: hidden [T, H] and weight [E, H] expected");
+  const int64_t T = hidden.size(0), H = hidden.size(1), E = weight.size(0);
+  TORCH_CHECK(indices.dim() == 2 && indices.size(0) == T && indices.scalar_type() == at::kLong,
+              "router_topk_backward: indices must be int64 [T, K]");
+  TORCH_CHECK(scores.dim() == 2 && scores.size(0) == T && scores.size(1) == E && d_scores.sizes() == scores.sizes(),
+              "router_topk_backward: scores and d_scores must be [T, E]");
+  TORCH_CHECK(weight.scalar_type() == hidden.scalar_type() && scores.scalar_type() == hidden.scalar_type() &&
+              d_scores.scalar_type() == hidden.scalar_type(), "router_topk_backward: one dtype for all float tensors");
+  const int code = dtype_code(hidden, "hidden");
+  at::Tensor x = hidden.contiguous(), w = weight.contiguous(), g = d_scores.contiguous(), sc = scores.contiguous(),
+             ix = indices.contiguous();
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(hidden.device());
+  at::Tensor d_hidden = at::empty_like(x), d_weight = at::empty_like(w), d_bias = at::empty({E}, hidden.options());
+  const size_t need = yamoe_router_backward_workspace_bytes((int)T, (int)E, code);
+  at::Tensor ws = at::empty({(int64_t)(need > 0 ? need : 1)}, hidden.options().dtype(at::kByte));
+  check_rc(yamoe_router_backward(g.data_ptr(), ix.data_ptr<int64_t>(), sc.data_ptr(), x.data_ptr(), w.data_ptr(), (int)T, (int)H,
+                                 (int)E, (int)indices.size(1), code, d_hidden.data_ptr(), d_weight.data_ptr(),
+                                 d_bias.data_ptr(), ws.data_ptr(), need, current_stream()),
+           "yamoe_router_backward");
+  return std::make_tuple(d_hidden, d_weight, d_bias);
+}
+
 }  // namespace
 
 TORCH_LIBRARY(_yamoe_amd_ops, ops) {
   ops.def("router_topk(Tensor hidden, Tensor weight, Tensor? bias, int top_k) -> (Tensor, Tensor)");
   ops.impl("router_topk", c10::DispatchKey::CUDA, &router_topk_op);
+  ops.def("router_topk_backward(Tensor d_scores, Tensor indices, Tensor scores, Tensor hidden, Tensor weight) -> "
+          "(Tensor, Tensor, Tensor)");
+  ops.impl("router_topk_backward", c10::DispatchKey::CUDA, &router_topk_backward_op);
   ops.def("gather(Tensor x, Tensor indices, Tensor bins, Tensor! output, int E, int C, int top_k) -> ()");
   ops.impl("gather", c10::DispatchKey::CUDA, &gather_op);
   ops.def("scatter(Tensor src, Tensor indices, Tensor bins, Tensor weights, Tensor! y, int T, int E, int C, "

@@ -40,10 +40,33 @@ def experts_autograd(hidden_flat, router_indices, routing_weights, gate_up_proj,
                             down_proj_bias, expert_capacity, num_experts, top_k, enable_router_grads)
 
 
-def router_kernel_takes(x_flat, weight, top_k):
-    """Shapes and dtypes of the fused router kernel (yamoe_router_topk)."""
-    return (x_flat.is_cuda and x_flat.dtype in (torch.bfloat16, torch.float16) and weight.dtype == x_flat.dtype
-            and x_flat.shape[1] % 16 == 0 and weight.shape[0] <= 256 and top_k <= min(16, weight.shape[0]))
+class _RouterFn(torch.autograd.Function):
+    """The fused router step with its gradient (yamoe_router_topk / yamoe_router_backward): what autograd gives through
+    the reference's linear -> topk -> softmax -> scatter_ (torch-ext/yamoe/layers.py:128-149), on the HIP kernels."""
+
+    @staticmethod
+    def forward(ctx, x_flat, weight, bias, top_k):
+        router_indices, router_scores = ops.router_topk(x_flat, weight, bias, top_k)
+        ctx.save_for_backward(x_flat, weight, router_indices, router_scores)
+        ctx.has_bias = bias is not None
+        ctx.mark_non_differentiable(router_indices)
+        return router_indices, router_scores
+
+    @staticmethod
+    def backward(ctx, _d_indices, d_scores):
+        x_flat, weight, router_indices, router_scores = ctx.saved_tensors
+        d_x, d_w, d_b = ops.router_topk_backward(d_scores.contiguous(), router_indices, router_scores, x_flat, weight)
+        return d_x, d_w, (d_b if ctx.has_bias else None), None
+
+
+def router_kernel_takes(x_flat, weight, top_k, with_grad=False):
+    """Shapes and dtypes of the fused router kernel (yamoe_router_topk) and, with_grad, of its gradient."""
+    step = 8 if x_flat.dtype == torch.float32 else 16
+    ok = (x_flat.is_cuda and x_flat.dtype in (torch.bfloat16, torch.float16, torch.float32) and weight.dtype == x_flat.dtype
+          and x_flat.shape[1] % step == 0 and weight.shape[0] <= 256 and top_k <= min(16, weight.shape[0]))
+    if with_grad:   # the two small products run on the expert GEMM kernels: 16-byte rows on both sides
+        ok = ok and weight.shape[0] % (step // 2) == 0
+    return ok
 
 
 class Yamoe(torch.nn.Module):
@@ -84,15 +107,19 @@ class Yamoe(torch.nn.Module):
             t0 = time.perf_counter()
         x_flat = hidden_states.reshape(-1, hidden)
         want_router_grads = torch.is_grad_enabled() and getattr(self, "enable_router_grads", False)
-        if router_kernel_takes(x_flat, self.router.weight, top_k) and not want_router_grads:
-            # linear + top-k + softmax + dense scatter in one kernel
-            router_indices, router_scores = ops.router_topk(x_flat, self.router.weight, self.router.bias, top_k)
+        if router_kernel_takes(x_flat, self.router.weight, top_k, with_grad=want_router_grads):
+            # linear + top-k + softmax + dense scatter in one kernel (and, for a router that is being trained, the
+            # gradient of the four steps on the HIP kernels as well)
+            if want_router_grads:
+                router_indices, router_scores = _RouterFn.apply(x_flat, self.router.weight, self.router.bias, top_k)
+            else:
+                router_indices, router_scores = ops.router_topk(x_flat, self.router.weight, self.router.bias, top_k)
             if timing:
                 t1 = lap("router", t0)
                 stats["topk_softmax"] = 0.0
         else:
-            # the same four steps as torch ops on the GPU (fp32 activations, shapes the kernel does not take, or a
-            # router that is being trained: autograd needs the chain)
+            # the same four steps as torch ops on the GPU, for shapes the kernels do not take (more than 256 experts,
+            # hidden sizes or, with gradients, expert counts that are not multiples of 16 bytes)
             logits = torch.nn.functional.linear(x_flat, self.router.weight, self.router.bias)
             if timing:
                 t1 = lap("router", t0)
