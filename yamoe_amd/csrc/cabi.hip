@@ -86,8 +86,9 @@ template <typename T>
 int gemm_async_dgrad(const void *, const int *, int, const void *, void *, const void *, int, int, int, int,
                      const void *, float *, hipStream_t);
 template <typename T>
-int gemm_async_wgrad(const void *, const int *, int, int, const void *, void *, const int *, const int *, int, int, int,
-                     int, hipStream_t);
+int gemm_async_wgrad(const void *, const int *, int, int, const void *, void *, void *, const int *, const int *, int, int,
+                     int, int, hipStream_t);
+bool wgrad_writes_bias(int Md, int Nd);
 bool gemm_async_supported(int Kd, int Nd, int lda, int ldb, long long a_span_bytes);
 bool gemm_f32_supported(int Kd, int Nd, int lda, int ldb, long long a_span_bytes);
 int gemm_f32_gate_up(const void *, const int *, const void *, const void *, void *, void *, const void *, int, int, int,
@@ -150,16 +151,23 @@ template <typename T> static bool wgrad_gathers(int Md, int Nd) {
   return false;
 }
 
+// True when the weight-gradient kernel for this dtype and shape also leaves the bias gradient (the per-expert column
+// sums of its right operand), so that no launch of expert_colsum_kernel is needed for it.
+template <typename T> static bool wgrad_sums_bias(int Md, int Nd) {
+  if constexpr (sizeof(T) == 2) return wgrad_writes_bias(Md, Nd);
+  return false;
+}
+
 // l_rows (with wgrad_gathers only): sorted row p of the left operand is row l_rows[p] / l_div of L; the list holds
-// n_rows values below n_rows and is followed by at least 32 readable ints
+// n_rows values below n_rows and is followed by at least 32 readable ints.  d_bias (with wgrad_sums_bias only): [E, Nd].
 template <typename T>
-static int tiles_wgrad(const void *L, const int *l_rows, int l_div, int n_rows, const void *R, void *dW,
+static int tiles_wgrad(const void *L, const int *l_rows, int l_div, int n_rows, const void *R, void *dW, void *d_bias,
                        const int *counts, const int *offsets, int capacity, int E, int Md, int Nd, hipStream_t stream) {
   if constexpr (sizeof(T) == 2) {
     if (wgrad_async_supported(Md, Nd))
-      return gemm_async_wgrad<T>(L, l_rows, l_div, n_rows, R, dW, counts, offsets, capacity, E, Md, Nd, stream);
+      return gemm_async_wgrad<T>(L, l_rows, l_div, n_rows, R, dW, d_bias, counts, offsets, capacity, E, Md, Nd, stream);
   }
-  if (l_rows != nullptr) { set_error("tiles_wgrad: this kernel takes its rows in expert order"); return YAMOE_E_ARG; }
+  if (l_rows != nullptr || d_bias != nullptr) { set_error("tiles_wgrad: this kernel takes its rows in expert order and sums no bias"); return YAMOE_E_ARG; }
   return gemm_wgrad<T>(L, R, dW, counts, offsets, capacity, E, Md, Nd, stream);
 }
 
@@ -338,27 +346,30 @@ static int backward_impl(const yamoe_problem *p, const void *gy, const void *x, 
                                        b.w_sorted, b.row_dot, N, p->K, E, H, stream));
   // down projection: bias and weight gradients from the weighted rows; the input gradient from the un-weighted
   // rows of grad_out, gathered by token (its dot with the activations is the rest of the routing gradient)
-  YAMOE_TRY(launch_expert_colsum<T>(b.g_y_perm, b.f.counts, b.f.offsets, cap, d_bd, E, H, stream));
+  // (the bias gradients are the column sums of the weight gradients' right operands: taken by those kernels where
+  // they can, by a launch of their own otherwise)
+  const bool bd_fused = wgrad_sums_bias<T>(I, H), bgu_fused = wgrad_sums_bias<T>(H, 2 * I);
+  if (!bd_fused) YAMOE_TRY(launch_expert_colsum<T>(b.g_y_perm, b.f.counts, b.f.offsets, cap, d_bd, E, H, stream));
   YAMOE_TRY(tiles_dgrad<T>(gy, b.f.sorted_idx, p->K, (long long)p->T * H * (long long)es, wd, b.d_act, b.f.schedule, N, E,
                            /*Kd=*/H, /*Nd=*/I, b.f.act, b.dot_part, stream));
-  YAMOE_TRY(tiles_wgrad<T>(b.f.act, nullptr, 1, 0, b.g_y_perm, d_wd, b.f.counts, b.f.offsets, cap, E, /*Md=*/I, /*Nd=*/H,
-                           stream));
+  YAMOE_TRY(tiles_wgrad<T>(b.f.act, nullptr, 1, 0, b.g_y_perm, d_wd, bd_fused ? d_bd : nullptr, b.f.counts, b.f.offsets, cap, E,
+                           /*Md=*/I, /*Nd=*/H, stream));
   // GLU backward (scaled by the routing weight) and the routing gradient
   YAMOE_TRY(glu_backward_rows<T>(b.d_act, b.pre, b.w_sorted, b.dot_part, b.n_part, b.f.sorted_idx, b.f.inv_pos, b.d_pre,
                                  b.row_dot, N, I, stream));
   YAMOE_TRY(launch_routing_grad<T>(b.row_dot, b.f.inv_pos, idx, p->idx_i64, p->rw_cols, d_rw, N, p->K, E, stream));
   // gate_up projection
-  YAMOE_TRY(launch_expert_colsum<T>(b.d_pre, b.f.counts, b.f.offsets, cap, d_bgu, E, 2 * I, stream));
+  if (!bgu_fused) YAMOE_TRY(launch_expert_colsum<T>(b.d_pre, b.f.counts, b.f.offsets, cap, d_bgu, E, 2 * I, stream));
   YAMOE_TRY(tiles_dgrad<T>(b.d_pre, nullptr, 1, 0, wgu, b.d_x_perm, b.f.schedule, N, E, /*Kd=*/2 * I, /*Nd=*/H, nullptr,
                            nullptr, stream));
   // (the hidden rows gathered by token where the kernel can do that; check_problem keeps hidden below 4 GiB, and
   // sorted_idx is followed in the workspace by inv_pos and the rest: readable well past its end)
   if (gathers)
-    YAMOE_TRY(tiles_wgrad<T>(x, b.f.sorted_idx, p->K, N, b.d_pre, d_wgu, b.f.counts, b.f.offsets, cap, E, /*Md=*/H,
-                             /*Nd=*/2 * I, stream));
+    YAMOE_TRY(tiles_wgrad<T>(x, b.f.sorted_idx, p->K, N, b.d_pre, d_wgu, bgu_fused ? d_bgu : nullptr, b.f.counts, b.f.offsets,
+                             cap, E, /*Md=*/H, /*Nd=*/2 * I, stream));
   else
-    YAMOE_TRY(tiles_wgrad<T>(b.x_perm, nullptr, 1, 0, b.d_pre, d_wgu, b.f.counts, b.f.offsets, cap, E, /*Md=*/H, /*Nd=*/2 * I,
-                             stream));
+    YAMOE_TRY(tiles_wgrad<T>(b.x_perm, nullptr, 1, 0, b.d_pre, d_wgu, bgu_fused ? d_bgu : nullptr, b.f.counts, b.f.offsets,
+                             cap, E, /*Md=*/H, /*Nd=*/2 * I, stream));
   // permute backward: d_hidden[t] = sum_k d_x_perm[inv_pos[t,k]]
   YAMOE_TRY(launch_combine<T>(b.d_x_perm, b.f.inv_pos, idx, p->idx_i64, nullptr, p->K, d_x, p->T, p->K, E, H, stream));
   return 0;

@@ -126,10 +126,12 @@ template <typename T> __device__ inline T pre_activation_store(float v, bool up)
 }
 
 // 16 bytes per lane from global memory straight into LDS at lds_base + lane * 16.
+// (lds_base is the same for every lane; saying so keeps it in a scalar register even where the compiler has merged
+// its computation with a per-lane address of the same LDS buffer)
 __device__ inline void copy16_to_lds(const void *uniform_base, uint32_t lane_byte_off, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
                :
-               : "v"(lane_byte_off), "s"(uniform_base), "s"(lds_base)
+               : "v"(lane_byte_off), "s"(uniform_base), "s"(__builtin_amdgcn_readfirstlane(lds_base))
                : "memory", "m0");
 }
 

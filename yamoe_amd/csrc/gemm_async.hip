@@ -752,6 +752,9 @@ struct WgradArgs {
   FastDiv a_div;
   int a_rows_max;  // largest value a_rows may hold
   int capacity, E, Md, Nd, n_m_tiles, n_n_tiles;
+  // optional: [E, Nd] column sums of the expert's rows of B (the bias gradient that goes with this weight gradient,
+  // csrc/experts_backward.cu:277, 308); needs Md % 128 != 0 (see wgrad_writes_bias)
+  void *bias_grad;
 };
 
 template <bool P1_, bool P2_, bool NEXT_, bool ZERO_, int VM_> struct WStepCfg {
@@ -769,9 +772,14 @@ constexpr int kSmallRing = kSmallStages * (kSmallAStage + kSmallBStage);
 constexpr int kSmallStaging = kSmallBM * (kBN * 2 + 16);
 constexpr int kSmallLds = kSmallRing > kSmallStaging ? kSmallRing : kSmallStaging;
 
+// bias_tile: this is the last row tile of the gradient and has room below its rows_m valid rows.  Column rows_m of the
+// left operand's LDS tile then holds 1 for every valid k (planted after each slab's copies have landed), so that row
+// rows_m of the product is 1^T . R, the column sums of the expert's rows of R: the bias gradient, taken by the same
+// MFMAs in fp32 instead of by a launch of its own over the same rows (17.5 + 37 us at the GPT-OSS-20B shape).
 template <typename T, int NMI, bool GATHER>
 __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid, const int expert, const int m0,
-                                            const int n0, const int rows_m, const long long first, const int rows) {
+                                            const int n0, const int rows_m, const long long first, const int rows,
+                                            const bool bias_tile) {
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
@@ -869,6 +877,16 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
     }
   };
 
+  // the ones column of slab `slab` (whose copies by this wave have landed): this wave's 8 k rows; lane l and the seven
+  // lanes l + 8 j write the same value to the same place (a branch on the lane number here would be the loop's only
+  // divergent one)
+  const int ones_k = 8 * wave + (lane & 7);
+  char *const ones_at = lds + ones_k * 256 + (((rows_m >> 3) ^ ((ones_k & 3) << 2)) << 4) + (rows_m & 7) * 2;
+  auto plant_ones = [&](int slab) {
+    if (bias_tile)
+      *(T *)(ones_at + (slab % kSmallStages) * kSmallAStage) = ElemTraits<T>::from_f32(slab * kBK + ones_k < rows ? 1.0f : 0.0f);
+  };
+
   const int g = lane >> 5, rl = lane & 31, j4 = (lane & 15) >> 2, q4 = lane & 3;
   int a_rd[NACC], b_rd[4];
 #pragma unroll
@@ -910,6 +928,7 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
       if (s < n_slabs) copy_slab(s);
     if (n_slabs >= 6) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");  // slab 0 is enough to start with
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    plant_ones(0);
 #pragma unroll
     for (int s = 0; s < kSmallStages; ++s)
       if (n_slabs < 6 && s < n_slabs && (s + 1) * kBK > rows) zero_tail(s);
@@ -975,6 +994,7 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
     }
     if constexpr (C::VM == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
     else if constexpr (C::VM == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if constexpr (C::NEXT) plant_ones(s + 1);
     if constexpr (C::ZERO) zero_tail(s + 1);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
@@ -1026,6 +1046,7 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
     }
     if constexpr (C::VM == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
     else if constexpr (C::VM == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if constexpr (C::NEXT) plant_ones(s + 1);
     if constexpr (C::ZERO) zero_tail(s + 1);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
@@ -1073,6 +1094,7 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
 #pragma unroll
       for (int j = 0; j < kMma; ++j) Mma<T>::run(fb0[j & 3], fa0[j >> 2], acc[j >> 2][j & 3]);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (s + 1 < n_slabs) plant_ones(s + 1);
       if (s + 1 < n_slabs && (s + 2) * kBK > rows) zero_tail(s + 1);
       __syncthreads();
       if (s + kSmallStages < n_slabs) copy_slab(s + kSmallStages);
@@ -1111,6 +1133,9 @@ __device__ inline void run_wgrad_tile_small(const WgradArgs &args, const int tid
         // operand tiles out of L2
         __builtin_nontemporal_store(*(const u32x4 *)(lds + r * stride + c * 16), (u32x4 *)(p + (long long)r * args.Nd));
       }
+      // the row below the valid ones: the column sums
+      if (bias_tile && tid < chunks)
+        *(u32x4 *)((T *)args.bias_grad + (long long)expert * args.Nd + n0 + c * 8) = *(const u32x4 *)(lds + rows_m * stride + c * 16);
     }
   }
 }
@@ -1128,15 +1153,17 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_small_kernel(const WgradArg
   const int expert = L / per_expert, r = L - expert * per_expert;
   const int n0 = (r / args.n_m_tiles) * kBN, m0 = (r % args.n_m_tiles) * kSmallBM;
   const int rows_m = min(kSmallBM, args.Md - m0);
-  int rows = min(args.counts[expert], args.capacity);
+  // (the same for every lane; said explicitly, so that the operand addresses built from them stay in scalar registers)
+  int rows = min(__builtin_amdgcn_readfirstlane(args.counts[expert]), args.capacity);
   if (rows < 0) rows = 0;
-  const long long first = args.offsets[expert];
-  const int n_blocks32 = (rows_m + 31) >> 5;
+  const long long first = __builtin_amdgcn_readfirstlane(args.offsets[expert]);
+  const bool bias_tile = args.bias_grad != nullptr && rows_m < kSmallBM;  // (the last row tile; see wgrad_writes_bias)
+  const int n_blocks32 = (rows_m + (bias_tile ? 1 : 0) + 31) >> 5;
   const int n_mi = (n_blocks32 - wm + 1) >> 1;
   switch (n_mi) {
-    case 2: run_wgrad_tile_small<T, 2, GATHER>(args, tid, expert, m0, n0, rows_m, first, rows); break;
-    case 1: run_wgrad_tile_small<T, 1, GATHER>(args, tid, expert, m0, n0, rows_m, first, rows); break;
-    default: run_wgrad_tile_small<T, 0, GATHER>(args, tid, expert, m0, n0, rows_m, first, rows); break;
+    case 2: run_wgrad_tile_small<T, 2, GATHER>(args, tid, expert, m0, n0, rows_m, first, rows, bias_tile); break;
+    case 1: run_wgrad_tile_small<T, 1, GATHER>(args, tid, expert, m0, n0, rows_m, first, rows, bias_tile); break;
+    default: run_wgrad_tile_small<T, 0, GATHER>(args, tid, expert, m0, n0, rows_m, first, rows, bias_tile); break;
   }
 }
 
@@ -1203,6 +1230,9 @@ int gemm_async_dgrad(const void *g, const int *g_rows, int g_div, const void *w,
 // dW[E, Md, Nd] = per expert L^T R over its kept rows.  Both operand buffers must stay readable for 32 rows past
 // their last row (the copies of a partial last slab run over; what they fetch is zeroed before use).
 bool wgrad_async_supported(int Md, int Nd) { return Md % 8 == 0 && Nd % 8 == 0; }
+// True when gemm_async_wgrad can leave the bias gradient (the column sums of the right operand's rows per expert) next
+// to the weight gradient: its last 128-row tile of the Md output rows must have a spare row.
+bool wgrad_writes_bias(int Md, int Nd) { return wgrad_async_supported(Md, Nd) && Md % async::kSmallBM != 0; }
 
 namespace async {
 template <typename T, bool GATHER> static int launch_wgrad(const WgradArgs &a, hipStream_t stream) {
@@ -1221,10 +1251,14 @@ template <typename T, bool GATHER> static int launch_wgrad(const WgradArgs &a, h
 // [n_rows / l_div, Md] tensor gathered by token, which must span less than 4 GiB); l_rows holds n_rows values below
 // n_rows and must stay readable for 32 values more, and L needs no readable rows past its end.
 template <typename T>
-int gemm_async_wgrad(const void *L, const int *l_rows, int l_div, int n_rows, const void *R, void *dW, const int *counts,
-                     const int *offsets, int capacity, int E, int Md, int Nd, hipStream_t stream) {
+int gemm_async_wgrad(const void *L, const int *l_rows, int l_div, int n_rows, const void *R, void *dW, void *d_bias,
+                     const int *counts, const int *offsets, int capacity, int E, int Md, int Nd, hipStream_t stream) {
+  if (d_bias != nullptr && !wgrad_writes_bias(Md, Nd)) {
+    set_error("gemm_async_wgrad: no spare row for the bias gradient at Md = %d", Md);
+    return YAMOE_E_ARG;
+  }
   async::WgradArgs a = {};
-  a.A = L; a.B = R; a.C = dW; a.counts = counts; a.offsets = offsets; a.capacity = capacity;
+  a.A = L; a.B = R; a.C = dW; a.counts = counts; a.offsets = offsets; a.capacity = capacity; a.bias_grad = d_bias;
   a.a_rows = l_rows; a.a_div = make_fast_div(l_rows != nullptr ? l_div : 1); a.a_rows_max = n_rows > 0 ? n_rows - 1 : 0;
   a.E = E; a.Md = Md; a.Nd = Nd;
   a.n_m_tiles = ceil_div(Md, async::kSmallBM);
@@ -1240,8 +1274,8 @@ int gemm_async_wgrad(const void *L, const int *l_rows, int l_div, int n_rows, co
                                   int, int, hipStream_t);                                                             \
   template int gemm_async_dgrad<T>(const void *, const int *, int, const void *, void *, const void *, int, int, int,  \
                                    int, const void *, float *, hipStream_t);                                           \
-  template int gemm_async_wgrad<T>(const void *, const int *, int, int, const void *, void *, const int *, const int *, \
-                                   int, int, int, int, hipStream_t);
+  template int gemm_async_wgrad<T>(const void *, const int *, int, int, const void *, void *, void *, const int *,     \
+                                   const int *, int, int, int, int, hipStream_t);
 YAMOE_INSTANTIATE_ASYNC(bf16_t)
 YAMOE_INSTANTIATE_ASYNC(f16_t)
 
