@@ -25,12 +25,14 @@ extern "C" {
 
 /* 2: YAMOE_F64 dtype code; yamoe_experts_forward_static; yamoe_route_workspace_bytes returns the size of a
  *    segments x buckets table above 4096 assignments (it was a constant 256 bytes); stream_max_rows up to 32;
- *    yamoe_probe_mfma_rate; yamoe_router_topk takes fp32; yamoe_router_backward. */
+ *    yamoe_probe_mfma_rate; yamoe_router_topk takes fp32; yamoe_router_backward; the whole op takes YAMOE_F64. */
 #define YAMOE_ABI_VERSION 2
 
-/* element type of activations, weights, biases and routing weights.  YAMOE_F64 is taken by the row movers among
- * the helper ops only (yamoe_padded_gather, yamoe_padded_scatter, yamoe_index_select), which the reference
- * dispatches over double too (csrc/gather.cu:89, csrc/scatter.cu:128); everything else answers YAMOE_E_DTYPE. */
+/* element type of activations, weights, biases and routing weights.  YAMOE_F64 is taken by the whole forward and
+ * backward (yamoe_experts_forward, _forward_static, _backward: plain FMA kernels, a compatibility dtype) and by the
+ * row movers among the helper ops (yamoe_padded_gather, yamoe_padded_scatter, yamoe_index_select), which the
+ * reference dispatches over double too (csrc/gather.cu:89, csrc/scatter.cu:128, csrc/experts_backward.cu:236);
+ * everything else answers YAMOE_E_DTYPE. */
 enum { YAMOE_F32 = 0, YAMOE_F16 = 1, YAMOE_BF16 = 2, YAMOE_F64 = 3 };
 
 enum {
@@ -48,7 +50,7 @@ typedef struct yamoe_problem {
   int32_t H;         /* hidden size */
   int32_t I;         /* intermediate size; gate_up_proj is [E,H,2I], down_proj is [E,I,H] */
   int32_t capacity;  /* expert_capacity: assignments ranked >= capacity inside their expert are dropped */
-  int32_t dtype;     /* YAMOE_F32 / YAMOE_F16 / YAMOE_BF16 */
+  int32_t dtype;     /* YAMOE_F32 / YAMOE_F16 / YAMOE_BF16 / YAMOE_F64 */
   int32_t idx_i64;   /* router_indices element type: 1 = int64, 0 = int32 */
   int32_t rw_cols;   /* columns of routing_weights: E (dense [T,E]) or K (per slot [T,K]) */
 } yamoe_problem;
@@ -120,7 +122,7 @@ int yamoe_down(const void *act, const void *down_proj, const void *down_proj_bia
                void *stream);
 
 /* ---- the whole forward: experts_cuda (csrc/moe.cpp:45-223) -------------------
- * Limits (YAMOE_E_ARG otherwise): H and I multiples of 8 (16-bit dtypes) or 4 (fp32); E <= 768;
+ * Limits (YAMOE_E_ARG otherwise): H and I multiples of 8 (16-bit dtypes) or 4 (fp32), any for fp64; E <= 768;
  * T*K < 2^30; hidden_states (and grad_out) below 4 GiB. */
 size_t yamoe_experts_workspace_bytes(const yamoe_problem *p);
 int yamoe_experts_forward(const yamoe_problem *p, const void *hidden_states,

@@ -13,8 +13,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libyamoe_hip.so")
 
 ABI_VERSION = 2   # YAMOE_ABI_VERSION of the header this module mirrors
-F32, F16, BF16 = 0, 1, 2
-_DTYPE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
+F32, F16, BF16, F64 = 0, 1, 2, 3
+_DTYPE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.float64: F64}
 
 # every symbol include/yamoe_hip.h declares
 SYMBOLS = [

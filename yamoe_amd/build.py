@@ -18,7 +18,7 @@ OBJ = os.path.join(HERE, "_obj")
 LIB_HIP = os.path.join(HERE, "libyamoe_hip.so")
 LIB_OPS = os.path.join(HERE, "_yamoe_amd_ops.so")
 
-HIP_SOURCES = ["route.hip", "permute.hip", "gemm.hip", "gemm_async.hip", "gemm_f32.hip", "stream.hip", "subops.hip", "router.hip", "probe.hip", "cabi.hip"]
+HIP_SOURCES = ["route.hip", "permute.hip", "gemm.hip", "gemm_async.hip", "gemm_f32.hip", "stream.hip", "subops.hip", "router.hip", "probe.hip", "f64.hip", "cabi.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall",
@@ -49,7 +49,7 @@ def build_hip(verbose=True):
                 print("\n".join(lines))
         return obj
 
-    with ThreadPoolExecutor(max_workers=min(10, len(HIP_SOURCES))) as ex:
+    with ThreadPoolExecutor(max_workers=min(11, len(HIP_SOURCES))) as ex:
         objs = list(ex.map(compile_one, HIP_SOURCES))
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_HIP] + objs)
     if verbose:

@@ -28,7 +28,8 @@ int dtype_code(const at::Tensor &t, const char *name) {
   return -1;
 }
 
-// the row movers among the helper ops also take float64, like the reference's (csrc/gather.cu:89, csrc/scatter.cu:128)
+// the whole op and the row movers among the helper ops also take float64, like the reference's
+// (AT_DISPATCH_FLOATING_TYPES_AND2: csrc/gather.cu:89, csrc/scatter.cu:128, csrc/experts_backward.cu:236)
 int mover_dtype_code(const at::Tensor &t, const char *name) {
   if (t.scalar_type() == at::kDouble) return YAMOE_F64;
   return dtype_code(t, name);
@@ -103,7 +104,7 @@ Checked check_inputs(const at::Tensor &hidden_states, const at::Tensor &router_i
   c.p.H = (int32_t)H;
   c.p.I = (int32_t)I;
   c.p.capacity = (int32_t)std::min<int64_t>(std::max<int64_t>(expert_capacity, 0), INT32_MAX);
-  c.p.dtype = dtype_code(hidden_states, "hidden_states");
+  c.p.dtype = mover_dtype_code(hidden_states, "hidden_states");
   c.p.idx_i64 = router_indices.scalar_type() == at::kLong ? 1 : 0;
   c.p.rw_cols = (int32_t)routing_weights.size(1);
   return c;
