@@ -7,7 +7,7 @@ stamps (gemm_async.hip compiled with -DYAMOE_TILE_STAMPS) and a run of the GPT-O
 Per tile the kernel leaves the shader clock at six points (workgroup entry, work-list look-ups done, first slab landed,
 contraction loop done, epilogue values staged, stores issued) plus its shape and the CU it ran on.  The summary gives, per
 tile shape, the median clocks of each phase and the loop's clocks per slab of 32 against the MFMA issue time of that
-shape, and over the launch the share of time each CU spent inside tiles.  The stamped build is a separate file; the
+shape, and over the launch the share of the longest CU's span that a CU spends inside tiles.  The stamped build is a separate file; the
 product library is not touched.
 """
 import ctypes
@@ -112,22 +112,28 @@ def run():
             issue = 2 * mi * ni * 32
             print("   %-22s %6d %8.0f %10.0f %8.0f %9.0f %7.0f %8.0f %12.0f %10d" % (
                 "%d (<= %d) x %d" % (r32, r32, c), cnt, ph[0], ph[1], ph[2], ph[3], ph[4], total, ph[2] / n_slabs, issue))
-        # the shader clock is a per-XCD counter: spans are taken XCD by XCD
+        # The counters of different CUs are not aligned with each other, so spans are taken CU by CU (first tile's entry
+        # to last tile's end); they tick at one rate, and the longest of them is, to a tile start, the launch itself.
         dur = (s[:, 5] - s[:, 0]).astype(np.float64)
-        xcc, cu = s[:, 7] >> 8, s[:, 7]
-        spans, busy, per = [], [], []
-        for x in np.unique(xcc):
-            m = xcc == x
-            span = float(s[m, 5].max() - s[m, 0].min())
-            spans.append(span)
-            for c in np.unique(cu[m]):
-                busy.append(dur[cu == c].sum() / span)
-                per.append(int((cu == c).sum()))
-        busy, per = np.array(busy), np.array(per)
-        print("   launch: %.0f clocks from an XCD's first tile entry to its last tile's end (mean of %d XCDs, %.0f .. %.0f); "
-              "%d CUs seen, %.1f tiles each (%d .. %d); a CU is inside tiles %.1f %% of its XCD's span on average (least busy "
-              "%.1f %%, busiest %.1f %%)" % (np.mean(spans), len(spans), min(spans), max(spans), len(busy), per.mean(),
-                                              per.min(), per.max(), 100 * busy.mean(), 100 * busy.min(), 100 * busy.max()))
+        cu = s[:, 7]
+        spans, inside, per = [], [], []
+        for c in np.unique(cu):
+            m = cu == c
+            spans.append(float(s[m, 5].max() - s[m, 0].min()))
+            inside.append(dur[m].sum())
+            per.append(int(m.sum()))
+        spans, inside, per = np.array(spans), np.array(inside), np.array(per)
+        launch = spans.max()
+        print("   launch: %d CUs seen, %.1f tiles each (%d .. %d); the longest CU span (first entry to last end) is %.0f clocks; "
+              "a CU is inside tiles %.1f %% of that on average (least busy %.1f %%, busiest %.1f %%) and %.1f %% of its own "
+              "span (the rest: between two tiles)" % (len(per), per.mean(), per.min(), per.max(), launch,
+                                                       100 * inside.mean() / launch, 100 * inside.min() / launch,
+                                                       100 * inside.max() / launch, 100 * (inside / spans).mean()))
+        xcc = s[:, 7] >> 8
+        per_xcd = np.array([dur[xcc == x].sum() for x in np.unique(xcc)])
+        cu_span_xcd = np.array([spans[[int(c) >> 8 == int(x) for c in np.unique(cu)]].max() for x in np.unique(xcc)])
+        print("   per XCD: tile clocks %s (mean = 100); longest CU span %s (longest = 100)" % (
+            " ".join("%.0f" % v for v in 100 * per_xcd / per_xcd.mean()), " ".join("%.0f" % v for v in 100 * cu_span_xcd / launch)))
         tot = dur.sum()
         parts = [(s[:, i + 1] - s[:, i]).astype(np.float64).sum() / tot for i in range(5)]
         print("   share of all tile clocks: look-ups %.1f %%, first slab %.1f %%, loop %.1f %%, epilogue %.1f %%, stores %.1f %%"
