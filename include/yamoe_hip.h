@@ -122,8 +122,10 @@ int yamoe_down(const void *act, const void *down_proj, const void *down_proj_bia
                void *stream);
 
 /* ---- the whole forward: experts_cuda (csrc/moe.cpp:45-223) -------------------
- * Limits (YAMOE_E_ARG otherwise): H and I multiples of 8 (16-bit dtypes) or 4 (fp32), any for fp64; E <= 768;
- * T*K < 2^30; hidden_states (and grad_out) below 4 GiB. */
+ * Limits (YAMOE_E_ARG otherwise): E <= 768; T*K < 2^30; hidden_states (and grad_out) below 4 GiB.
+ * H and I may be any size, as in the reference; the MFMA kernels take those that are whole 16-byte chunks (multiples
+ * of 8 for the 16-bit dtypes, of 4 for fp32), and every other size, like every fp64 problem, runs on plain FMA tiles
+ * (correct to the same tolerances, far slower). */
 size_t yamoe_experts_workspace_bytes(const yamoe_problem *p);
 int yamoe_experts_forward(const yamoe_problem *p, const void *hidden_states,
                           const void *router_indices, const void *routing_weights,

@@ -38,8 +38,11 @@ def test_size_queries_and_validation_need_no_gpu():
     assert fwd >= n * 2880 * 2 * 2 and bwd > fwd            # act + y_perm at least
     assert fwd < 2 * n * 2880 * 2 * 2                       # and nothing padded to [E, C, *]
     assert lib.yamoe_schedule_bytes(n, 32) % 256 == 0
-    # rejected shapes: H not a multiple of the 16-byte vector, routing weights with a wrong width, bad dtype
-    for bad in (dict(H=2881), dict(rw_cols=7), dict(dtype=9), dict(K=0)):
+    # a hidden size that is not a whole 16-byte chunk is accepted (it runs on the plain-FMA kernels)
+    q = _cabi.Problem(**{**{f: getattr(p, f) for f, _ in p._fields_}, **dict(H=2881)})
+    assert lib.yamoe_experts_workspace_bytes(ctypes.byref(q)) > 0
+    # rejected shapes: routing weights with a wrong width, bad dtype, no slots
+    for bad in (dict(rw_cols=7), dict(dtype=9), dict(K=0)):
         q = _cabi.Problem(**{**{f: getattr(p, f) for f, _ in p._fields_}, **bad})
         assert lib.yamoe_experts_workspace_bytes(ctypes.byref(q)) == 0
         assert len(lib.yamoe_last_error()) > 0

@@ -18,7 +18,7 @@ OBJ = os.path.join(HERE, "_obj")
 LIB_HIP = os.path.join(HERE, "libyamoe_hip.so")
 LIB_OPS = os.path.join(HERE, "_yamoe_amd_ops.so")
 
-HIP_SOURCES = ["route.hip", "permute.hip", "gemm.hip", "gemm_async.hip", "gemm_f32.hip", "stream.hip", "subops.hip", "router.hip", "probe.hip", "f64.hip", "cabi.hip"]
+HIP_SOURCES = ["route.hip", "permute.hip", "gemm.hip", "gemm_async.hip", "gemm_f32.hip", "stream.hip", "subops.hip", "router.hip", "probe.hip", "plain.hip", "cabi.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall",

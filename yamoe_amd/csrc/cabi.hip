@@ -99,14 +99,16 @@ bool wgrad_async_supported(int Md, int Nd);
 template <typename T>
 int launch_router_backward_logits(const void *, const long long *, const void *, int, int, int, void *, hipStream_t);
 
-// the double-precision path (f64.hip)
-int f64_forward(const void *, const void *, int, const void *, int, const void *, const void *, const void *, const void *,
-                void *, const int *, const int *, const void *, void *, void *, int, int, int, int, int, hipStream_t);
-int f64_backward(const void *, const void *, const void *, int, const void *, int, const void *, const void *, const void *,
-                 const void *, void *, void *, void *, void *, void *, void *, const int *, const int *, const int *,
-                 const int *, const int *, const void *, void *, void *, void *, void *, void *, void *, void *, void *, int,
-                 int, int, int, int, int, hipStream_t);
-int f64_fill_zero(void *, long long, hipStream_t);
+// the plain-FMA path (plain.hip): double precision, and sizes that are not whole 16-byte chunks
+template <typename T>
+int plain_forward(const void *, const void *, int, const void *, int, const void *, const void *, const void *, const void *,
+                  void *, const int *, const int *, const void *, void *, void *, int, int, int, int, int, hipStream_t);
+template <typename T>
+int plain_backward(const void *, const void *, const void *, int, const void *, int, const void *, const void *, const void *,
+                   const void *, void *, void *, void *, void *, void *, void *, const int *, const int *, const int *,
+                   const int *, const int *, const void *, void *, void *, void *, void *, void *, void *, void *, void *, int,
+                   int, int, int, int, int, hipStream_t);
+template <typename T> int plain_fill_zero(void *, long long, hipStream_t);
 
 template <typename T> struct HasStreamPath { static constexpr bool value = sizeof(T) == 2; };
 
@@ -203,11 +205,6 @@ static int check_problem(const yamoe_problem *p, const char *who) {
   if (p->dtype != YAMOE_F32 && p->dtype != YAMOE_F16 && p->dtype != YAMOE_BF16 && p->dtype != YAMOE_F64) {
     set_error("%s: unknown dtype %d", who, p->dtype);
     return YAMOE_E_DTYPE;
-  }
-  int vec = p->dtype == YAMOE_F64 ? 1 : 16 / (int)dtype_size(p->dtype);  // (the double-precision kernels move single elements)
-  if (p->H % vec != 0 || p->I % vec != 0) {
-    set_error("%s: H and I must be multiples of %d for this dtype (H=%d I=%d)", who, vec, p->H, p->I);
-    return YAMOE_E_ARG;
   }
   if (p->rw_cols != p->E && p->rw_cols != p->K) {
     set_error("%s: routing_weights must be [T,E] or [T,K] (got %d columns, E=%d K=%d)", who, p->rw_cols, p->E, p->K);
@@ -384,8 +381,16 @@ static int backward_impl(const yamoe_problem *p, const void *gy, const void *x, 
   return 0;
 }
 
-// double precision: the same lists, then the kernels of f64.hip
-static int forward_f64(const yamoe_problem *p, const void *x, const void *idx, const void *rw, const void *wgu,
+// Double precision, and hidden or intermediate sizes that are not whole 16-byte chunks (the unit the MFMA kernels
+// copy): the same lists, then the kernels of plain.hip.
+static bool takes_plain_path(const yamoe_problem *p) {
+  if (p->dtype == YAMOE_F64) return true;
+  const int vec = 16 / (int)dtype_size(p->dtype);
+  return p->H % vec != 0 || p->I % vec != 0;
+}
+
+template <typename T>
+static int forward_plain(const yamoe_problem *p, const void *x, const void *idx, const void *rw, const void *wgu,
                        const void *bgu, const void *wd, const void *bd, void *out, void *ws, hipStream_t stream) {
   ForwardBuffers b;
   carve_forward(p, ws, &b);
@@ -393,28 +398,29 @@ static int forward_f64(const yamoe_problem *p, const void *x, const void *idx, c
   if (N == 0 || p->T == 0) return 0;
   YAMOE_TRY(route_and_schedule(idx, p->idx_i64, N, p->E, p->capacity, b.sorted_expert, b.sorted_idx, b.counts, b.offsets,
                                b.inv_pos, b.route_ws, b.route_ws_bytes, 0, b.schedule, b.schedule_bytes, (void *)stream));
-  return f64_forward(x, idx, p->idx_i64, rw, p->rw_cols, wgu, bgu, wd, bd, out, b.sorted_idx, b.inv_pos, b.schedule, b.act,
+  return plain_forward<T>(x, idx, p->idx_i64, rw, p->rw_cols, wgu, bgu, wd, bd, out, b.sorted_idx, b.inv_pos, b.schedule, b.act,
                      b.y_perm, p->T, p->K, p->E, p->H, p->I, stream);
 }
 
-static int backward_f64(const yamoe_problem *p, const void *gy, const void *x, const void *idx, const void *rw,
+template <typename T>
+static int backward_plain(const yamoe_problem *p, const void *gy, const void *x, const void *idx, const void *rw,
                         const void *wgu, const void *bgu, const void *wd, const void *bd, void *d_x, void *d_rw, void *d_wgu,
                         void *d_bgu, void *d_wd, void *d_bd, void *ws, hipStream_t stream) {
   BackwardBuffers b;
   carve_backward(p, ws, &b);
   const int N = p->T * p->K, E = p->E, H = p->H, I = p->I, cap = p->capacity < 0 ? 0 : p->capacity;
   if (N == 0) {
-    YAMOE_TRY(f64_fill_zero(d_rw, (long long)p->T * p->rw_cols, stream));
-    YAMOE_TRY(f64_fill_zero(d_wgu, (long long)E * H * 2 * I, stream));
-    YAMOE_TRY(f64_fill_zero(d_bgu, (long long)E * 2 * I, stream));
-    YAMOE_TRY(f64_fill_zero(d_wd, (long long)E * I * H, stream));
-    YAMOE_TRY(f64_fill_zero(d_bd, (long long)E * H, stream));
+    YAMOE_TRY(plain_fill_zero<T>(d_rw, (long long)p->T * p->rw_cols, stream));
+    YAMOE_TRY(plain_fill_zero<T>(d_wgu, (long long)E * H * 2 * I, stream));
+    YAMOE_TRY(plain_fill_zero<T>(d_bgu, (long long)E * 2 * I, stream));
+    YAMOE_TRY(plain_fill_zero<T>(d_wd, (long long)E * I * H, stream));
+    YAMOE_TRY(plain_fill_zero<T>(d_bd, (long long)E * H, stream));
     return 0;
   }
   YAMOE_TRY(route_and_schedule(idx, p->idx_i64, N, E, cap, b.f.sorted_expert, b.f.sorted_idx, b.f.counts, b.f.offsets,
                                b.f.inv_pos, b.f.route_ws, b.f.route_ws_bytes, 0, b.f.schedule, b.f.schedule_bytes,
                                (void *)stream));
-  return f64_backward(gy, x, idx, p->idx_i64, rw, p->rw_cols, wgu, bgu, wd, bd, d_x, d_rw, d_wgu, d_bgu, d_wd, d_bd,
+  return plain_backward<T>(gy, x, idx, p->idx_i64, rw, p->rw_cols, wgu, bgu, wd, bd, d_x, d_rw, d_wgu, d_bgu, d_wd, d_bd,
                       b.f.sorted_expert, b.f.sorted_idx, b.f.inv_pos, b.f.counts, b.f.offsets, b.f.schedule, b.f.act, b.pre,
                       b.g_y_perm, b.d_act, b.d_pre, b.d_x_perm, b.w_sorted, b.row_dot, p->T, p->K, E, H, I, cap, stream);
 }
@@ -422,6 +428,15 @@ static int backward_f64(const yamoe_problem *p, const void *gy, const void *x, c
 }  // namespace yamoe
 
 using namespace yamoe;
+
+#define YAMOE_DISPATCH_ALL(dtype, CALL)                                   \
+  switch (dtype) {                                                        \
+    case YAMOE_F64: { typedef double T; return CALL; }                    \
+    case YAMOE_F32: { typedef float T; return CALL; }                     \
+    case YAMOE_BF16: { typedef bf16_t T; return CALL; }                   \
+    case YAMOE_F16: { typedef f16_t T; return CALL; }                     \
+    default: set_error("unknown dtype %d", dtype); return YAMOE_E_DTYPE;  \
+  }
 
 #define YAMOE_DISPATCH(dtype, CALL)                                       \
   switch (dtype) {                                                        \
@@ -516,9 +531,11 @@ extern "C" int yamoe_experts_forward(const yamoe_problem *p, const void *hidden_
     set_error("yamoe_experts_forward: workspace too small (%zu < %zu)", workspace_bytes, need);
     return YAMOE_E_WORKSPACE;
   }
-  if (p->dtype == YAMOE_F64)
-    return forward_f64(p, hidden_states, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
-                       down_proj_bias, out, workspace, (hipStream_t)stream);
+  if (takes_plain_path(p)) {
+    YAMOE_DISPATCH_ALL(p->dtype, forward_plain<T>(p, hidden_states, router_indices, routing_weights, gate_up_proj,
+                                                  gate_up_proj_bias, down_proj, down_proj_bias, out, workspace,
+                                                  (hipStream_t)stream));
+  }
   YAMOE_DISPATCH(p->dtype, forward_impl<T>(p, hidden_states, router_indices, routing_weights, gate_up_proj,
                                            gate_up_proj_bias, down_proj, down_proj_bias, out, workspace,
                                            (hipStream_t)stream));
@@ -574,9 +591,11 @@ extern "C" int yamoe_experts_forward_static(const yamoe_problem *p, const void *
   YAMOE_TRY(static_scratch(&ws));
   // Nothing in the workspace has to start at zero: every list, counter and row the kernels read is written earlier
   // in the same call, so the contents left by the previous call on this GPU do not matter.
-  if (p->dtype == YAMOE_F64)
-    return forward_f64(p, hidden_states, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
-                       down_proj_bias, out, ws, (hipStream_t)stream);
+  if (takes_plain_path(p)) {
+    YAMOE_DISPATCH_ALL(p->dtype, forward_plain<T>(p, hidden_states, router_indices, routing_weights, gate_up_proj,
+                                                  gate_up_proj_bias, down_proj, down_proj_bias, out, ws,
+                                                  (hipStream_t)stream));
+  }
   YAMOE_DISPATCH(p->dtype, forward_impl<T>(p, hidden_states, router_indices, routing_weights, gate_up_proj,
                                            gate_up_proj_bias, down_proj, down_proj_bias, out, ws, (hipStream_t)stream));
 }
@@ -605,10 +624,12 @@ extern "C" int yamoe_experts_backward(const yamoe_problem *p, const void *grad_o
     set_error("yamoe_experts_backward: workspace too small (%zu < %zu)", workspace_bytes, need);
     return YAMOE_E_WORKSPACE;
   }
-  if (p->dtype == YAMOE_F64)
-    return backward_f64(p, grad_out, hidden_states, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias,
-                        down_proj, down_proj_bias, d_hidden, d_routing, d_gate_up_proj, d_gate_up_proj_bias, d_down_proj,
-                        d_down_proj_bias, workspace, (hipStream_t)stream);
+  if (takes_plain_path(p)) {
+    YAMOE_DISPATCH_ALL(p->dtype, backward_plain<T>(p, grad_out, hidden_states, router_indices, routing_weights, gate_up_proj,
+                                                   gate_up_proj_bias, down_proj, down_proj_bias, d_hidden, d_routing,
+                                                   d_gate_up_proj, d_gate_up_proj_bias, d_down_proj, d_down_proj_bias,
+                                                   workspace, (hipStream_t)stream));
+  }
   YAMOE_DISPATCH(p->dtype, backward_impl<T>(p, grad_out, hidden_states, router_indices, routing_weights, gate_up_proj,
                                             gate_up_proj_bias, down_proj, down_proj_bias, d_hidden, d_routing,
                                             d_gate_up_proj, d_gate_up_proj_bias, d_down_proj, d_down_proj_bias,
