@@ -76,6 +76,24 @@ def test_forward_partial_column_tiles(gpu, dtype, rows):
     assert report("partial column tiles", got, want, REL_L2_TOL[dtype]) < REL_L2_TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows", [3841, 4096, 4400, 6200, 8192])
+def test_forward_experts_with_many_row_tiles(gpu, dtype, rows):
+    """An expert with sixteen or more row tiles is walked in bands of eight row tiles (the last band takes the remainder:
+    3841 and 4096 rows are bands of 8 + 8 tiles, 4400 of 8 + 10, 6200 of 8 + 8 + 9, 8192 of four 8s), next to one that
+    is walked column by column (300 rows); three and two column tiles, the last partial."""
+    H, I = 576, 320
+    T = rows + 300
+    d = make_inputs(T, H, I, 3, 1, dtype, seed=rows, w_std=0.05, bias_std=0.1)
+    idx = torch.zeros(T, 1, dtype=torch.int64)
+    idx[rows:] = 2                                   # expert 1 stays empty
+    idx = idx[torch.randperm(T, generator=torch.Generator().manual_seed(rows))]
+    d["router_indices"] = idx
+    got = run_op(d, T, gpu)
+    want = oracle_forward(d, T)
+    assert report("many row tiles", got, want, REL_L2_TOL[dtype]) < REL_L2_TOL[dtype]
+
+
 def test_forward_uneven_tile_costs(gpu):
     """Eight experts with 2048 rows each and 56 experts with 20 rows each: the shares of the tile list that the
     8 XCDs get are equal in cost, so the shares made of small tiles hold more tiles than the grid has workgroups
