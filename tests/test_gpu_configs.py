@@ -71,3 +71,34 @@ def test_zipf_shape_forward(gpu):
     torch.cuda.empty_cache()
     want = oracle_forward(d, c["T"])
     assert report("zipf 16384 tokens", got, want, 1e-2) < 1e-2
+
+
+@pytest.mark.parametrize("tokens,experts", [(65536, 32), (16384, 128)])
+def test_token_order_does_not_change_a_row_at_scale(gpu, tokens, experts):
+    """Beyond the sizes the oracle is run at: 65 536 tokens on 32 experts (8192 rows per expert, every expert walked in
+    bands of row tiles) and 16 384 tokens with Zipf routing on 128 experts, H = I = 2880, top-4, bf16.  A token's output
+    depends on its own row only, and the kernels add a row's products in an order that does not depend on where the row
+    sits in a tile: the same tokens in another order must give the same bits, row for row.  Spot rows are checked
+    against the oracle."""
+    import yamoe_amd
+    from yamoe_amd.workloads import make_routing
+    H = I = 2880
+    K = 4
+    gen = torch.Generator().manual_seed(tokens)
+    idx, dense = make_routing(tokens, experts, K, gen, zipf=1.2 if experts == 128 else 0.0)
+    x = (torch.randn(tokens, H, generator=gen)).to(torch.bfloat16)
+    w = device_weights(experts, H, I, torch.bfloat16, 0.02, 9, gpu)
+    dense = dense.to(torch.bfloat16)
+    perm = torch.randperm(tokens, generator=gen)
+    a = (w["gate_up_proj"], w["gate_up_proj_bias"], w["down_proj"], w["down_proj_bias"], tokens, experts, K)
+    out = yamoe_amd.experts(x.to(gpu), idx.to(gpu), dense.to(gpu), *a)
+    out_p = yamoe_amd.experts(x[perm].to(gpu), idx[perm].to(gpu), dense[perm].to(gpu), *a)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    assert torch.equal(out[perm.to(gpu)], out_p)
+    # 64 spot tokens against the oracle (their rows of the batch alone: a token's output needs no other token)
+    spot = torch.randperm(tokens, generator=gen)[:64]
+    d = dict(hidden=x[spot], router_indices=idx[spot], routing_weights=dense[spot],
+             **{k: v.cpu() for k, v in w.items()})
+    want = oracle_forward(d, 64)
+    assert report("spot rows of %d tokens" % tokens, out[spot.to(gpu)].cpu(), want, 1e-2) < 1e-2
