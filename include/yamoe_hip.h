@@ -108,6 +108,10 @@ int yamoe_combine(const void *y_perm, const int32_t *inv_pos, const void *router
  * listed for the weight-streaming kernel, the others are cut into 256-row MFMA tiles.
  * A limit above 16 applies only when no expert has more kept rows than the limit;
  * otherwise experts with up to 16 rows stream and the others are tiled.
+ * stream_max_rows = -1 with N <= 4*E (decode: a few rows per expert) lists every expert for the
+ * streaming kernel, one with more than 32 rows as several entries of at most 32, and leaves the
+ * tile list empty (the whole-op forward then skips the tile kernels' launches); with more
+ * assignments than that -1 means 32.
  * yamoe_gate_up / yamoe_down launch both kernels; each walks its own list. */
 size_t yamoe_schedule_bytes(int32_t N, int32_t E);
 int yamoe_build_schedule(const int32_t *counts, const int32_t *offsets, int32_t N, int32_t E,

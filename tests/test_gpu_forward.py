@@ -94,6 +94,23 @@ def test_forward_experts_with_many_row_tiles(gpu, dtype, rows):
     assert report("many row tiles", got, want, REL_L2_TOL[dtype]) < REL_L2_TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,E,K,hot", [(100, 32, 1, 70), (64, 128, 4, 0), (128, 40, 1, 100), (33, 9, 1, 33)])
+def test_forward_every_expert_streams(gpu, dtype, T, E, K, hot):
+    """At most 4 assignments per expert on average: every expert goes through the streaming kernel, an expert with
+    more than 32 rows in chunks of 32 (`hot` tokens are sent to expert 3: 70 rows are chunks of 32 + 32 + 6, 100 of
+    32 + 32 + 32 + 4, 33 of 32 + 1), and the tile kernels are not launched."""
+    H, I = 192, 160
+    d = make_inputs(T, H, I, E, K, dtype, seed=T + E, w_std=0.05, bias_std=0.1)
+    assert T * K <= 4 * E
+    if hot:
+        d["router_indices"][:hot, 0] = 3
+        d["routing_weights"] = torch.rand(T, E, generator=torch.Generator().manual_seed(1)).to(dtype)
+    got = run_op(d, T, gpu)
+    want = oracle_forward(d, T)
+    assert report("every expert streams", got, want, REL_L2_TOL[dtype]) < REL_L2_TOL[dtype]
+
+
 def test_forward_uneven_tile_costs(gpu):
     """Eight experts with 2048 rows each and 56 experts with 20 rows each: the shares of the tile list that the
     8 XCDs get are equal in cost, so the shares made of small tiles hold more tiles than the grid has workgroups

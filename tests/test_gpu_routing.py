@@ -112,9 +112,13 @@ def test_permute_and_combine(gpu, dtype, T, K, E, H):
                                                (1000, 700, 5, 0), (40, 3, 40, 16),
                                                (300, 40, 30, 32),      # every expert within 32 rows: all of them stream
                                                (300, 40, 300, 32),     # some beyond 32: the limit falls back to 16
-                                               (2000, 64, 32, 32)])    # capacity 32 keeps everybody within the limit
+                                               (2000, 64, 32, 32),     # capacity 32 keeps everybody within the limit
+                                               (256, 128, 256, -1),    # decode: everything streams, in chunks of 32 rows
+                                               (160, 40, 160, -1),     # the same with experts of several chunks
+                                               (2000, 64, 2000, -1)])  # too many assignments for that: as with 32
 def test_schedule_lists(gpu, N, E, C, stream_rows):
-    """The device-built work lists: experts with 1..stream_rows kept rows in the streaming list, the
+    """The device-built work lists: experts with 1..stream_rows kept rows in the streaming list (with -1 and few
+    assignments: every expert, in chunks of 32 rows), the
     rest cut into equal row tiles (as few as 256 rows allow, each a multiple of 32 rows but the last), both in
     expert order, none dropped, none duplicated.  A limit above 16 holds only if no expert exceeds it; with such
     experts present the limit is 16."""
@@ -127,14 +131,20 @@ def test_schedule_lists(gpu, N, E, C, stream_rows):
     offsets = torch.from_numpy(r["offsets"]).to(gpu)
     sched = _cabi.build_schedule(counts, offsets, N, C, stream_rows).cpu().numpy()
     want_tiles, want_small = [], []
-    if stream_rows > 16 and int(np.minimum(r["counts"], C).max()) > stream_rows:
+    # -1: every expert streams, in chunks of 32 rows, if there are at most 4 assignments per expert on average
+    everything = stream_rows == -1 and N <= 4 * E
+    if stream_rows == -1:
+        stream_rows = 32
+    if not everything and stream_rows > 16 and int(np.minimum(r["counts"], C).max()) > stream_rows:
         stream_rows = 16
     for e in range(E):
         kept = min(int(r["counts"][e]), C)
         if kept == 0:
             continue
         first = int(r["offsets"][e])
-        if kept <= stream_rows:
+        if everything:
+            want_small += [(e, first + c, min(32, kept - c)) for c in range(0, kept, 32)]
+        elif kept <= stream_rows:
             want_small.append((e, first, kept))
         else:
             g0, n = len(want_tiles), -(-kept // 256)

@@ -306,10 +306,15 @@ static int forward_impl(const yamoe_problem *p, const void *x, const void *idx, 
   void *st = (void *)stream;
   if (N == 0 || p->T == 0) return 0;
   const int stream_rows = HasStreamPath<T>::value ? kStreamMaxRows : 0;
+  // At most 4 assignments per expert on average (decode): every expert goes to the streaming kernel, in chunks of
+  // stream_rows rows where one has more, and the tile kernels, whose lists are then empty, are not launched (two
+  // launches of 4.5 us each that found nothing to do at 64 tokens on 128 experts).
+  const bool everything = HasStreamPath<T>::value && sched_may_stream_everything(N, p->E);
   YAMOE_TRY(route_and_schedule(idx, p->idx_i64, N, p->E, p->capacity, b.sorted_expert, b.sorted_idx, b.counts, b.offsets,
-                               b.inv_pos, b.route_ws, b.route_ws_bytes, stream_rows, b.schedule, b.schedule_bytes, st));
-  // with no more assignments than a streamed expert may have rows, every expert is streamed: the tile lists are empty
-  const bool tiles = N > stream_rows;
+                               b.inv_pos, b.route_ws, b.route_ws_bytes, everything ? kStreamEverything : stream_rows,
+                               b.schedule, b.schedule_bytes, st));
+  // with no more assignments than a streamed expert may have rows, every expert is streamed as well
+  const bool tiles = !everything && N > stream_rows;
   if (tiles)
     YAMOE_TRY(tiles_gate_up<T>(x, b.sorted_idx, wgu, bgu, b.act, nullptr, b.schedule, N, p->K, p->E, p->H, p->I, stream_rows,
                                stream));

@@ -187,7 +187,14 @@ __host__ __device__ inline int sched_grid_row_tiles(int N, int E, int small_rows
   if (tiled > E) tiled = E;
   return N / kRowTile + tiled + 1;
 }
-__host__ __device__ inline int sched_max_small(int N, int E) { return (N < E ? N : E) + 1; }
+// Every expert may be put on the streaming list in chunks of at most kStreamMaxRows rows (stream_max_rows =
+// kStreamEverything) when there are at most 4 assignments per expert on average: the weights of an expert with more
+// rows than one chunk are then read once per chunk, which is rare at that load, and the tile kernels are not launched.
+constexpr int kStreamEverything = -1;
+__host__ __device__ inline bool sched_may_stream_everything(int N, int E) { return N <= 4 * E; }
+__host__ __device__ inline int sched_max_small(int N, int E) {
+  return (N < E ? N : E) + (sched_may_stream_everything(N, E) ? N / kStreamMaxRows : 0) + 1;
+}
 
 struct ScheduleView {
   const int *hdr;

@@ -152,7 +152,9 @@ __device__ inline void build_schedule_wave(const int *counts, const int *offsets
   // Experts of 17 to 32 rows stream only when every expert streams: next to experts that need the tile kernels anyway
   // they are better off as tiles (two half-filled launches one after the other are slower than one: 0.35 against
   // 0.31 ms for 32 experts of about 32 rows, where 0.27 against 0.31 ms is gained when all of them have at most 32).
-  if (stream_max_rows > kStreamMixedRows) {
+  const bool everything = stream_max_rows == kStreamEverything;  // (the host checked sched_may_stream_everything)
+  if (everything) stream_max_rows = kStreamMaxRows;
+  if (!everything && stream_max_rows > kStreamMixedRows) {
     int most = 0;
     for (int base = 0; base < E; base += kWave) {
       int e = base + lane;
@@ -167,16 +169,17 @@ __device__ inline void build_schedule_wave(const int *counts, const int *offsets
     int kept = e < E ? min(counts[e], capacity) : 0;
     if (kept < 0) kept = 0;
     int first = e < E ? offsets[e] : 0;
-    int is_small = kept > 0 && kept <= stream_max_rows;
+    // entries on the streaming list: one, or with `everything` one per chunk of kStreamMaxRows rows
+    int is_small = everything ? ceil_div(kept, kStreamMaxRows) : (kept > 0 && kept <= stream_max_rows);
     int tiles = (kept > 0 && !is_small) ? ceil_div(kept, kRowTile) : 0;
     int tot_small, tot_tiles, tot_active, tot_kept;
     int pos_small = wave_exclusive_scan(is_small, lane, tot_small);
     int pos_tiles = wave_exclusive_scan(tiles, lane, tot_tiles);
     wave_exclusive_scan(kept > 0 ? 1 : 0, lane, tot_active);
     wave_exclusive_scan(kept, lane, tot_kept);
-    if (is_small) {
-      int *s = small + 4 * (n_small + pos_small);
-      s[0] = e; s[1] = first; s[2] = kept; s[3] = 0;
+    for (int c = 0; c < is_small; ++c) {
+      int *s = small + 4 * (n_small + pos_small + c);
+      s[0] = e; s[1] = first + c * kStreamMaxRows; s[2] = min(kStreamMaxRows, kept - c * kStreamMaxRows); s[3] = 0;
     }
     int gfirst = n_tiles + pos_tiles;
     // An expert's rows are cut into equal tiles (a multiple of 32 rows, the MFMA block), not into full
@@ -200,7 +203,7 @@ __device__ inline void build_schedule_wave(const int *counts, const int *offsets
       int e = base + lane;
       int kept = e < E ? min(counts[e], capacity) : 0;
       if (kept < 0) kept = 0;
-      int is_small = kept > 0 && kept <= stream_max_rows;
+      int is_small = everything || (kept > 0 && kept <= stream_max_rows);
       int tiles = (kept > 0 && !is_small) ? ceil_div(kept, kRowTile) : 0;
       int per_tile = tiles > 0 ? min(kRowTile, (ceil_div(kept, tiles) + 31) & ~31) : 0;
       int w = sched_group_weight(tiles, per_tile, kept);
@@ -523,7 +526,8 @@ int yamoe::route_and_schedule(const void *router_indices, int32_t idx_i64, int32
     set_error("yamoe_build_schedule: schedule region too small");
     return YAMOE_E_WORKSPACE;
   }
-  if (stream_max_rows < 0) stream_max_rows = 0;
+  if (stream_max_rows == kStreamEverything && !sched_may_stream_everything(N, E)) stream_max_rows = kStreamMaxRows;
+  if (stream_max_rows < 0 && stream_max_rows != kStreamEverything) stream_max_rows = 0;
   if (stream_max_rows > kStreamMaxRows) stream_max_rows = kStreamMaxRows;
   if (N < 0 || E <= 0 || E + 1 > kRouteMaxBuckets) {
     set_error("yamoe_route: need N >= 0 and 1 <= E < %d (got N=%d E=%d)", kRouteMaxBuckets, N, E);
@@ -630,7 +634,8 @@ extern "C" int yamoe_build_schedule(const int32_t *counts, const int32_t *offset
     return YAMOE_E_WORKSPACE;
   }
   if (capacity < 0) capacity = 0;
-  if (stream_max_rows < 0) stream_max_rows = 0;
+  if (stream_max_rows == kStreamEverything && !sched_may_stream_everything(N, E)) stream_max_rows = kStreamMaxRows;
+  if (stream_max_rows < 0 && stream_max_rows != kStreamEverything) stream_max_rows = 0;
   if (stream_max_rows > kStreamMaxRows) stream_max_rows = kStreamMaxRows;
   hipLaunchKernelGGL(build_schedule_kernel, dim3(1), dim3(kWave), 0, stream, counts, offsets, N, E, capacity,
                      stream_max_rows, (int *)schedule);
