@@ -147,3 +147,21 @@ def test_hub_layout_imports_as_yamoe(tmp_path):
             "assert 'yamoe_amd' not in sys.modules; print('ok')" % os.path.dirname(dst))
     r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, cwd=str(tmp_path))
     assert r.returncode == 0 and r.stdout.strip().endswith("ok"), r.stderr[-2000:]
+
+
+def test_operators_answer_shape_queries_without_a_gpu():
+    """torch.compile and FakeTensorMode ask an operator what it returns without running it: meta tensors through the
+    functional operators give the shapes and dtypes the kernels would."""
+    import yamoe_amd
+    T, H, I, E, K = 12, 64, 48, 4, 2
+    m = lambda *shape, dtype=torch.bfloat16: torch.empty(*shape, dtype=dtype, device="meta")
+    x, idx, rw = m(T, H), m(T, K, dtype=torch.int64), m(T, E)
+    w = (m(E, H, 2 * I), m(E, 2 * I), m(E, I, H), m(E, H))
+    out = yamoe_amd.experts(x, idx, rw, *w, T, E, K)
+    assert out.shape == (T, H) and out.dtype == torch.bfloat16 and out.device.type == "meta"
+    grads = yamoe_amd.experts_backward(m(T, H), x, idx, rw, *w, T, E, K)
+    assert [tuple(g.shape) for g in grads] == [(T, H), (T, E), (E, H, 2 * I), (E, 2 * I), (E, I, H), (E, H)]
+    indices, scores = yamoe_amd.router_topk(x, m(E, H), m(E), K)
+    assert indices.shape == (T, K) and indices.dtype == torch.int64 and scores.shape == (T, E)
+    d_hidden, d_weight, d_bias = yamoe_amd.router_topk_backward(scores, indices, scores, x, m(E, H))
+    assert d_hidden.shape == (T, H) and d_weight.shape == (E, H) and d_bias.shape == (E,)

@@ -51,3 +51,30 @@ def test_packaged_tree_runs_the_op(gpu, tmp_path):
     want_g = O.experts_backward(got["gy"], *[d[k] for k in KEYS], T, compute_dtype=torch.float32)
     for a, b in zip(got["grads"], want_g):
         assert O.rel_l2(a, b) < 1e-2
+
+
+def test_operators_trace_under_torch_compile(gpu):
+    """The operators carry shape functions, so a graph capture (torch.compile with the ahead-of-time eager backend: no
+    code generation, just the traced graph run operator by operator) goes through `experts_autograd` forward and
+    backward in one graph and gives the bits of the eager call."""
+    import yamoe_amd
+    from tests.util import args, to_dev
+    from yamoe_amd.workloads import make_inputs
+    T, H, I, E, K = 300, 128, 64, 4, 2
+    d = to_dev(make_inputs(T, H, I, E, K, torch.bfloat16, seed=5, w_std=0.2, bias_std=0.1), gpu)
+    leaves = [d[k].clone().requires_grad_(True) for k in ("hidden", "routing_weights", "gate_up_proj", "gate_up_proj_bias",
+                                                          "down_proj", "down_proj_bias")]
+
+    def forward(x, rw, wgu, bgu, wd, bd):
+        return yamoe_amd.experts_autograd(x, d["router_indices"], rw, wgu, bgu, wd, bd, T, E, K)
+
+    def step(fn):
+        out = fn(*leaves)
+        return out, torch.autograd.grad(out.float().square().sum(), leaves)
+
+    want_out, want_grads = step(forward)
+    got_out, got_grads = step(torch.compile(forward, backend="aot_eager", fullgraph=True))
+    torch.cuda.synchronize()
+    assert torch.equal(got_out, want_out)
+    for a, b in zip(got_grads, want_grads):
+        assert torch.equal(a, b)

@@ -28,3 +28,35 @@ for _name in ("experts", "experts_backward", "gather", "scatter", "sort", "binco
 
 def add_op_namespace_prefix(op_name: str) -> str:
     return "_yamoe_amd_ops::" + op_name
+
+
+# Shapes and dtypes of the outputs for tracing (torch.compile, FakeTensorMode, meta tensors): the kernels themselves run
+# on the GPU only, but a graph capture must be able to ask what an operator returns without running it.
+def _register_fakes():
+    fake = torch.library.register_fake
+
+    @fake("_yamoe_amd_ops::experts")
+    def _(hidden_states, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj, down_proj_bias,
+          expert_capacity, num_experts, top_k):
+        return hidden_states.new_empty(hidden_states.shape)
+
+    @fake("_yamoe_amd_ops::experts_backward")
+    def _(grad_out, hidden_states, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
+          down_proj_bias, expert_capacity, num_experts, top_k):
+        return [t.new_empty(t.shape) for t in (hidden_states, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
+                                               down_proj_bias)]
+
+    @fake("_yamoe_amd_ops::router_topk")
+    def _(hidden, weight, bias, top_k):
+        T, E = hidden.shape[0], weight.shape[0]
+        return hidden.new_empty((T, top_k), dtype=torch.int64), hidden.new_empty((T, E))
+
+    @fake("_yamoe_amd_ops::router_topk_backward")
+    def _(d_scores, indices, scores, hidden, weight):
+        return hidden.new_empty(hidden.shape), weight.new_empty(weight.shape), hidden.new_empty((weight.shape[0],))
+
+    for name in ("gather", "scatter", "sort", "bincount_cumsum"):  # these write into their output arguments
+        fake("_yamoe_amd_ops::" + name)(lambda *args, **kwargs: None)
+
+
+_register_fakes()
