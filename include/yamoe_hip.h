@@ -126,7 +126,10 @@ int yamoe_down(const void *act, const void *down_proj, const void *down_proj_bia
                void *stream);
 
 /* ---- the whole forward: experts_cuda (csrc/moe.cpp:45-223) -------------------
- * Limits (YAMOE_E_ARG otherwise): E <= 768; T*K < 2^30; hidden_states (and grad_out) below 4 GiB.
+ * Limits (YAMOE_E_ARG otherwise): E <= 768; T*K < 2^30.
+ * hidden_states (and grad_out) of 4 GiB or more are permuted into expert order first (the kernels gather token
+ * rows with 32-bit byte offsets from the start of the tensor): the workspace then holds one more [T*K, H] buffer
+ * (two for the backward).  yamoe_gate_up, the stage entry point, keeps the 4 GiB limit for its gathered x.
  * H and I may be any size, as in the reference; the MFMA kernels take those that are whole 16-byte chunks (multiples
  * of 8 for the 16-bit dtypes, of 4 for fp32), and every other size, like every fp64 problem, runs on plain FMA tiles
  * (correct to the same tolerances, far slower). */

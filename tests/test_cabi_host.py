@@ -46,14 +46,19 @@ def test_size_queries_and_validation_need_no_gpu():
         q = _cabi.Problem(**{**{f: getattr(p, f) for f, _ in p._fields_}, **bad})
         assert lib.yamoe_experts_workspace_bytes(ctypes.byref(q)) == 0
         assert len(lib.yamoe_last_error()) > 0
-    # hidden_states of 4 GiB or more: token rows are gathered with 32-bit byte offsets from the tensor's start
-    for T_big, dt, ok in ((745000, _cabi.BF16, True), (746000, _cabi.BF16, False), (372000, _cabi.F32, True),
-                          (373000, _cabi.F32, False)):
+    # hidden_states of 4 GiB or more: accepted; the workspace then holds the rows in expert order as well (the kernels
+    # gather token rows with 32-bit byte offsets from the tensor's start, so such a tensor is permuted first)
+    for T_big, dt, wide in ((745000, _cabi.BF16, False), (746000, _cabi.BF16, True), (372000, _cabi.F32, False),
+                            (373000, _cabi.F32, True)):
         q = _cabi.Problem(**{**{f: getattr(p, f) for f, _ in p._fields_}, **dict(T=T_big, capacity=T_big, dtype=dt)})
-        assert (lib.yamoe_experts_workspace_bytes(ctypes.byref(q)) > 0) == ok, (T_big, dt)
-        if not ok:
-            assert b"4 GiB" in lib.yamoe_last_error()
-            assert lib.yamoe_experts_backward_workspace_bytes(ctypes.byref(q)) == 0
+        es = 2 if dt == _cabi.BF16 else 4
+        n = T_big * 4
+        base = n * 2880 * es * 2                                   # act + y_perm
+        need = lib.yamoe_experts_workspace_bytes(ctypes.byref(q))
+        assert base < need < base + n * 2880 * es * (1 if wide else 0) + n * 64, (T_big, dt, need)
+        if wide:
+            assert need > base + n * 2880 * es
+        assert lib.yamoe_experts_backward_workspace_bytes(ctypes.byref(q)) > need
     rc = lib.yamoe_gate_up(None, None, None, None, None, None, None, 746000 * 4, 4, 32, 2880, 2880, _cabi.BF16, None)
     assert rc == -1
     # yamoe_route rejects too many experts before any launch

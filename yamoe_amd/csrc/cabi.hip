@@ -6,6 +6,7 @@
 
 #include <atomic>
 
+#include <cstdlib>
 #include "common.h"
 
 namespace yamoe {
@@ -117,16 +118,20 @@ template <typename T> struct HasStreamPath { static constexpr bool value = sizeo
 template <typename T>
 // `small_rows`: experts with at most this many kept rows are on the schedule's streaming list, not tiled (0 when
 // unknown); it only tightens the grid.
+// sorted_idx == nullptr: x holds one row per sorted row, in order (the callers permute a hidden_states tensor of 4 GiB or
+// more first: the kernels address gathered rows with 32-bit byte offsets from the start of the tensor).
 static int tiles_gate_up(const void *x, const int *sorted_idx, const void *w, const void *bias, void *act, void *pre,
                          const void *sched, int N, int K, int E, int H, int I, int small_rows, hipStream_t stream) {
+  const long long span = sorted_idx != nullptr ? (long long)(N / K) * H * (long long)sizeof(T) : 0;
   if constexpr (sizeof(T) == 2) {
     // the gathered source rows span the whole hidden_states tensor: N / K tokens of H elements
-    if (gemm_async_supported(H, 2 * I, H, 2 * I, (long long)(N / K) * H * (long long)sizeof(T)))
+    if (gemm_async_supported(H, 2 * I, H, 2 * I, span))
       return gemm_async_gate_up<T>(x, sorted_idx, w, bias, act, pre, sched, N, K, E, H, I, small_rows, stream);
   } else {
-    if (gemm_f32_supported(H, 2 * I, H, 2 * I, (long long)(N / K) * H * (long long)sizeof(T)))
+    if (gemm_f32_supported(H, 2 * I, H, 2 * I, span))
       return gemm_f32_gate_up(x, sorted_idx, w, bias, act, pre, sched, N, K, E, H, I, stream);
   }
+  if (span >= (1ll << 32)) { set_error("tiles_gate_up: gathered rows span 4 GiB or more"); return YAMOE_E_ARG; }
   return gemm_gate_up<T>(x, sorted_idx, w, bias, act, pre, sched, N, K, E, H, I, stream);
 }
 template <typename T>
@@ -152,6 +157,7 @@ static int tiles_dgrad(const void *g, const int *g_rows, int g_div, long long g_
     if (gemm_async_supported(Kd, Nd, Kd, Kd, g_rows ? g_span_bytes : 0))
       return gemm_async_dgrad<T>(g, g_rows, g_div, w, out, sched, N, E, Kd, Nd, dot_with, dot_part, stream);
   }
+  if (g_rows != nullptr && g_span_bytes >= (1ll << 32)) { set_error("tiles_dgrad: gathered rows span 4 GiB or more"); return YAMOE_E_ARG; }
   return gemm_dgrad<T>(g, g_rows, g_div, w, out, sched, N, E, Kd, Nd, dot_with, dot_part, stream);
 }
 
@@ -214,12 +220,21 @@ static int check_problem(const yamoe_problem *p, const char *who) {
     set_error("%s: T*K too large", who);
     return YAMOE_E_ARG;
   }
-  // the GEMM kernels address gathered token rows with 32-bit byte offsets from the start of the tensor
-  if ((long long)p->T * p->H * (long long)dtype_size(p->dtype) >= (1ll << 32)) {
-    set_error("%s: hidden_states / grad_out of 4 GiB or more are not supported (T=%d H=%d)", who, p->T, p->H);
-    return YAMOE_E_ARG;
-  }
   return 0;
+}
+
+// The GEMM kernels address gathered token rows (hidden_states in the gate_up product and its weight gradient, grad_out
+// in the input gradient of the down projection) with 32-bit byte offsets from the start of the tensor.  A tensor of
+// 4 GiB or more is permuted into expert order first (one more [N, H] buffer each, one more launch that moves
+// 2 * N * H elements) and read in order.  YAMOE_GATHER_SPAN_BYTES lowers the limit (the tests use it to run this path
+// at small sizes).
+static bool gathers_need_permute(const yamoe_problem *p) {
+  long long limit = 1ll << 32;
+  if (const char *e = getenv("YAMOE_GATHER_SPAN_BYTES")) {
+    const long long v = atoll(e);
+    if (v > 0 && v < limit) limit = v;
+  }
+  return (long long)p->T * p->H * (long long)dtype_size(p->dtype) >= limit;
 }
 
 // Carves 256-byte aligned regions out of the workspace.
@@ -237,6 +252,7 @@ struct Carver {
 struct ForwardBuffers {
   int *sorted_expert, *sorted_idx, *inv_pos, *counts, *offsets;
   void *schedule, *route_ws, *act, *y_perm;
+  void *x_perm;  // hidden rows in expert order: only with gathers_need_permute
   size_t schedule_bytes, route_ws_bytes;
 };
 
@@ -255,12 +271,14 @@ static size_t carve_forward(const yamoe_problem *p, void *ws, ForwardBuffers *b)
   b->act = c.take(N * p->I * es);
   // sized for the larger of H and I: the backward reuses this region for d_act [N, I]
   b->y_perm = c.take(N * (size_t)(p->H > p->I ? p->H : p->I) * es);
+  b->x_perm = gathers_need_permute(p) ? c.take(N * p->H * es) : nullptr;
   return c.used;
 }
 
 struct BackwardBuffers {
   ForwardBuffers f;
   void *x_perm, *pre, *g_y_perm, *d_act, *d_pre, *d_x_perm;
+  void *gy_perm;  // grad_out rows in expert order, un-weighted: only with gathers_need_permute
   float *w_sorted, *row_dot, *dot_part;
   int n_part;
 };
@@ -270,8 +288,10 @@ static size_t carve_backward(const yamoe_problem *p, void *ws, BackwardBuffers *
   const size_t N = (size_t)p->T * p->K, es = dtype_size(p->dtype);
   Carver c(ws ? (char *)ws + used : nullptr);
   // hidden rows in expert order: only where the gate_up weight-gradient kernel cannot gather them itself
-  const bool gathers = es == 2 ? wgrad_gathers<bf16_t>(p->H, 2 * p->I) : wgrad_gathers<float>(p->H, 2 * p->I);
-  b->x_perm = gathers ? nullptr : c.take(N * p->H * es);
+  const bool gathers = !gathers_need_permute(p) &&
+                       (es == 2 ? wgrad_gathers<bf16_t>(p->H, 2 * p->I) : wgrad_gathers<float>(p->H, 2 * p->I));
+  b->x_perm = gathers ? nullptr : b->f.x_perm != nullptr ? b->f.x_perm : c.take(N * p->H * es);
+  b->gy_perm = gathers_need_permute(p) ? c.take(N * p->H * es) : nullptr;
   b->pre = c.take(N * 2 * p->I * es);
   b->g_y_perm = c.take(N * p->H * es);
   b->d_pre = c.take(N * 2 * p->I * es);
@@ -315,9 +335,14 @@ static int forward_impl(const yamoe_problem *p, const void *x, const void *idx, 
                                b.schedule, b.schedule_bytes, st));
   // with no more assignments than a streamed expert may have rows, every expert is streamed as well
   const bool tiles = !everything && N > stream_rows;
-  if (tiles)
+  if (tiles && b.x_perm != nullptr) {  // (a hidden_states tensor too large to gather from: see gathers_need_permute)
+    YAMOE_TRY(launch_permute<T>(x, b.sorted_idx, b.x_perm, N, p->K, p->H, stream));
+    YAMOE_TRY(tiles_gate_up<T>(b.x_perm, nullptr, wgu, bgu, b.act, nullptr, b.schedule, N, p->K, p->E, p->H, p->I, stream_rows,
+                               stream));
+  } else if (tiles) {
     YAMOE_TRY(tiles_gate_up<T>(x, b.sorted_idx, wgu, bgu, b.act, nullptr, b.schedule, N, p->K, p->E, p->H, p->I, stream_rows,
                                stream));
+  }
   if constexpr (HasStreamPath<T>::value)
     YAMOE_TRY(stream_gate_up<T>(x, b.sorted_idx, wgu, bgu, b.act, nullptr, b.schedule, N, p->K, p->E, p->H, p->I,
                                 stream));
@@ -349,9 +374,13 @@ static int backward_impl(const yamoe_problem *p, const void *gy, const void *x, 
   YAMOE_TRY(route_and_schedule(idx, p->idx_i64, N, E, cap, b.f.sorted_expert, b.f.sorted_idx, b.f.counts, b.f.offsets,
                                b.f.inv_pos, b.f.route_ws, b.f.route_ws_bytes, 0, b.f.schedule, b.f.schedule_bytes, st));
   // forward recompute of the first product only: activations and pre-activations
-  const bool gathers = wgrad_gathers<T>(H, 2 * I);
+  const bool permuted = b.gy_perm != nullptr;  // hidden_states and grad_out too large to gather from
+  const bool gathers = !permuted && wgrad_gathers<T>(H, 2 * I);
   if (!gathers) YAMOE_TRY(launch_permute<T>(x, b.f.sorted_idx, b.x_perm, N, p->K, H, stream));
-  YAMOE_TRY(tiles_gate_up<T>(x, b.f.sorted_idx, wgu, bgu, b.f.act, b.pre, b.f.schedule, N, p->K, E, H, I, 0, stream));
+  if (permuted)
+    YAMOE_TRY(tiles_gate_up<T>(b.x_perm, nullptr, wgu, bgu, b.f.act, b.pre, b.f.schedule, N, p->K, E, H, I, 0, stream));
+  else
+    YAMOE_TRY(tiles_gate_up<T>(x, b.f.sorted_idx, wgu, bgu, b.f.act, b.pre, b.f.schedule, N, p->K, E, H, I, 0, stream));
   // combine backward: g_y_perm = grad_out[tok] * w, and the bias part of the routing gradient
   YAMOE_TRY(launch_combine_backward<T>(gy, bd, b.f.sorted_idx, b.f.inv_pos, idx, p->idx_i64, rw, p->rw_cols, b.g_y_perm,
                                        b.w_sorted, b.row_dot, N, p->K, E, H, stream));
@@ -361,8 +390,14 @@ static int backward_impl(const yamoe_problem *p, const void *gy, const void *x, 
   // they can, by a launch of their own otherwise)
   const bool bd_fused = wgrad_sums_bias<T>(I, H), bgu_fused = wgrad_sums_bias<T>(H, 2 * I);
   if (!bd_fused) YAMOE_TRY(launch_expert_colsum<T>(b.g_y_perm, b.f.counts, b.f.offsets, cap, d_bd, E, H, stream));
-  YAMOE_TRY(tiles_dgrad<T>(gy, b.f.sorted_idx, p->K, (long long)p->T * H * (long long)es, wd, b.d_act, b.f.schedule, N, E,
-                           /*Kd=*/H, /*Nd=*/I, b.f.act, b.dot_part, stream));
+  if (permuted) {
+    YAMOE_TRY(launch_permute<T>(gy, b.f.sorted_idx, b.gy_perm, N, p->K, H, stream));
+    YAMOE_TRY(tiles_dgrad<T>(b.gy_perm, nullptr, 1, 0, wd, b.d_act, b.f.schedule, N, E, /*Kd=*/H, /*Nd=*/I, b.f.act,
+                             b.dot_part, stream));
+  } else {
+    YAMOE_TRY(tiles_dgrad<T>(gy, b.f.sorted_idx, p->K, (long long)p->T * H * (long long)es, wd, b.d_act, b.f.schedule, N, E,
+                             /*Kd=*/H, /*Nd=*/I, b.f.act, b.dot_part, stream));
+  }
   YAMOE_TRY(tiles_wgrad<T>(b.f.act, nullptr, 1, 0, b.g_y_perm, d_wd, bd_fused ? d_bd : nullptr, b.f.counts, b.f.offsets, cap, E,
                            /*Md=*/I, /*Nd=*/H, stream));
   // GLU backward (scaled by the routing weight) and the routing gradient
@@ -373,8 +408,8 @@ static int backward_impl(const yamoe_problem *p, const void *gy, const void *x, 
   if (!bgu_fused) YAMOE_TRY(launch_expert_colsum<T>(b.d_pre, b.f.counts, b.f.offsets, cap, d_bgu, E, 2 * I, stream));
   YAMOE_TRY(tiles_dgrad<T>(b.d_pre, nullptr, 1, 0, wgu, b.d_x_perm, b.f.schedule, N, E, /*Kd=*/2 * I, /*Nd=*/H, nullptr,
                            nullptr, stream));
-  // (the hidden rows gathered by token where the kernel can do that; check_problem keeps hidden below 4 GiB, and
-  // sorted_idx is followed in the workspace by inv_pos and the rest: readable well past its end)
+  // (the hidden rows gathered by token where the kernel can do that and hidden_states is below 4 GiB; sorted_idx is
+  // followed in the workspace by inv_pos and the rest: readable well past its end)
   if (gathers)
     YAMOE_TRY(tiles_wgrad<T>(x, b.f.sorted_idx, p->K, N, b.d_pre, d_wgu, bgu_fused ? d_bgu : nullptr, b.f.counts, b.f.offsets,
                              cap, E, /*Md=*/H, /*Nd=*/2 * I, stream));

@@ -485,10 +485,11 @@ __global__ __launch_bounds__(kGemmThreads) void grouped_gemm_kernel(const GemmAr
       // byte offsets fit 32 bits: rows of a tile are near its first row, and gathered sources are
       // checked on the host to span less than 4 GB
       long long src = r;
-      if (GATHER) src = args.a_rows[ti.row0 + r] / args.a_div;
+      if (GATHER && args.a_rows != nullptr) src = args.a_rows[ti.row0 + r] / args.a_div;
       la.row_off[i] = (uint32_t)((src * args.lda + (tid & 7) * V) * (long long)sizeof(T));
     }
-    la.base = (const char *)((const T *)args.A + (GATHER ? 0ll : (long long)ti.row0 * args.lda));
+    // (a gathering instantiation without a row list reads its rows in order: see gemm_async.hip)
+    la.base = (const char *)((const T *)args.A + (GATHER && args.a_rows != nullptr ? 0ll : (long long)ti.row0 * args.lda));
   } else {
     la.setup((const T *)args.A + ti.a_first * args.lda + ti.m0, args.lda, lane & 7, wave * 8 + (lane >> 3), ti.k_len,
              ti.rows_valid);

@@ -654,6 +654,9 @@ __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
   }
 
   // A copies: copy i fetches rows 32*i + 8*wave + (lane >> 3); LDS position lane & 7 holds piece pos ^ ((row >> 1) & 7)
+  // (a gathering instantiation without a row list reads its rows in order, like the others: the form the callers use
+  // when the gathered tensor is too large for 32-bit byte offsets from its start and they have permuted it first)
+  const bool gathers = GATHER && args.a_rows != nullptr;
   uint32_t a_off[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -661,10 +664,10 @@ __global__ __launch_bounds__(kThreads) void gemm_async_kernel(const Args args) {
     int piece = (lane & 7) ^ ((row >> 1) & 7);
     int r = min(row, ti.rows_valid - 1);
     long long src = r;
-    if (GATHER) src = fast_div(args.a_rows[ti.row0 + r], args.a_div);
+    if (gathers) src = fast_div(args.a_rows[ti.row0 + r], args.a_div);
     a_off[i] = (uint32_t)((src * args.lda + piece * 8) * (long long)sizeof(T));
   }
-  const char *a_base = (const char *)((const T *)args.A + (GATHER ? 0ll : (long long)ti.row0 * args.lda));
+  const char *a_base = (const char *)((const T *)args.A + (gathers ? 0ll : (long long)ti.row0 * args.lda));
 
   const long long b_ld_bytes = (long long)args.ldb * (long long)sizeof(T);
   uint32_t b_off[8];

@@ -90,6 +90,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_kernel(const Args args) 
   // ---- copies.  A: copy i (0..3) fetches rows 32*i + 8*wave + (lane >> 3), 16 bytes of each; LDS position
   // lane & 7 of the row holds piece pos ^ ((row >> 1) & 7).  B: copy i fetches k rows 8*wave + 2*i + (lane >> 5),
   // piece lane & 31 (no swizzle: a half wave reads 256 contiguous bytes of one k row).
+  // (a gathering instantiation without a row list reads its rows in order: see gemm_async.hip)
+  const bool gathers = GATHER && args.a_rows != nullptr;
   uint32_t a_off[4], b_off[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -97,14 +99,14 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_kernel(const Args args) 
     const int piece = (lane & 7) ^ ((row >> 1) & 7);
     const int r = min(row, rows_valid - 1);  // rows past the end re-read the last one; never stored
     long long src = r;
-    if (GATHER) src = args.a_rows[row0 + r] / args.a_div;
+    if (gathers) src = args.a_rows[row0 + r] / args.a_div;
     a_off[i] = (uint32_t)((src * args.lda + piece * 4) * 4);
     const int k = 8 * wave + 2 * i + (lane >> 5);
     int col = (lane & 31) * 4;
     if (col >= cols_valid) col = 0;  // columns past the end re-read valid ones; never stored
     b_off[i] = (uint32_t)(((long long)k * args.ldb + col) * 4);
   }
-  const char *a_base = (const char *)(args.A + (GATHER ? 0ll : (long long)row0 * args.lda));
+  const char *a_base = (const char *)(args.A + (gathers ? 0ll : (long long)row0 * args.lda));
   const char *b_base = (const char *)(args.B + (long long)expert * args.b_expert_stride + n0);
   const long long b_slab_bytes = (long long)kBK * args.ldb * 4;
   const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds);
