@@ -352,3 +352,46 @@ def test_router_is_differentiable_and_picks_override():
     idx2, scores2, _ = O.router(x, w, b, 3, compute_dtype=torch.float64, picks=idx)
     assert torch.equal(idx, idx2) and torch.equal(scores, scores2)
     assert torch.autograd.gradcheck(lambda a, c, d: O.router(a, c, d, 3, compute_dtype=torch.float64, picks=idx)[1], (x, w, b))
+
+
+def test_torch_baselines_of_the_package_agree_with_the_oracle():
+    """yamoe_amd.reference / yamoe_amd.vendored (plain torch, for users to compare the operators against) give what the
+    oracle gives: the GPT-OSS modules in training and in inference form, the router, and the capacity-binned formulation
+    with and without drops and with dense and per-slot weights."""
+    import types
+
+    import yamoe_amd
+    from yamoe_amd.workloads import make_inputs
+    T, H, I, E, K = 90, 32, 24, 6, 2
+    d = make_inputs(T, H, I, E, K, torch.float64, seed=3, w_std=0.3, bias_std=0.2, zipf=0.7)
+    a = [d[k] for k in ("hidden", "router_indices", "routing_weights", "gate_up_proj", "gate_up_proj_bias", "down_proj",
+                        "down_proj_bias")]
+    for cap in (T, 11):
+        want = O.experts_capacity(*a, cap)
+        got = yamoe_amd.yamoe_ref.binned_experts_ref(*a, cap)
+        assert O.rel_l2(got, want) < 1e-13
+        per_slot = torch.gather(d["routing_weights"], 1, d["router_indices"])
+        got = yamoe_amd.vendored.yamoe_ref.binned_experts_ref(a[0].reshape(3, 30, H), a[1], per_slot, *a[3:], cap)
+        assert got.shape == (3, 30, H) and O.rel_l2(got.reshape(T, H), want) < 1e-13
+    cfg = types.SimpleNamespace(hidden_size=H, intermediate_size=I, num_local_experts=E, num_experts_per_tok=K)
+    mlp = yamoe_amd.gpt_oss_mlp.GptOssMLP(cfg).double()
+    assert yamoe_amd.reference.GptOssExperts is yamoe_amd.vendored.gpt_oss_mlp.GptOssExperts
+    with torch.no_grad():
+        for p, v in zip(mlp.experts.parameters(), a[3:]):
+            p.copy_(v)
+        mlp.router.weight.copy_(torch.randn(E, H, dtype=torch.float64, generator=torch.Generator().manual_seed(1)))
+        mlp.router.bias.copy_(torch.randn(E, dtype=torch.float64, generator=torch.Generator().manual_seed(2)))
+    out, scores = mlp(d["hidden"])
+    idx, want_scores, _ = O.router(d["hidden"], mlp.router.weight.detach(), mlp.router.bias.detach(), K,
+                                   compute_dtype=torch.float64)
+    assert O.rel_l2(scores.detach(), want_scores) < 1e-13
+    want = O.experts_loop(d["hidden"], idx, want_scores, *a[3:])
+    assert O.rel_l2(out.detach(), want) < 1e-13
+    # the dense form (what the module does in inference mode off the CPU), called directly
+    ex = mlp.experts
+    every = d["hidden"].unsqueeze(0).expand(E, -1, -1)
+    from yamoe_amd.torch_baseline import clamped_swiglu
+    rows = torch.bmm(clamped_swiglu(torch.bmm(every, ex.gate_up_proj) + ex.gate_up_proj_bias.unsqueeze(1)), ex.down_proj)
+    rows = rows + ex.down_proj_bias.unsqueeze(1)
+    dense = (rows * want_scores.t().unsqueeze(-1)).sum(0)
+    assert O.rel_l2(dense.detach(), want) < 1e-13

@@ -3,12 +3,16 @@
 Same surface as the reference package for this path (torch-ext/yamoe/__init__.py:1-12):
 `experts`, `experts_backward`, `gather`, `scatter`, `sort`, `bincount_cumsum`, `batch_mm`, `ops`, `Yamoe`.  Everything runs in hand-written HIP kernels behind
 the C ABI of libyamoe_hip.so; the first use of any of them fails if the native libraries are not built.
+`reference`, `vendored`, `yamoe_ref` and `gpt_oss_mlp` (torch-ext/yamoe/__init__.py:3-4, 29-31) are plain-torch baselines
+to compare against (torch_baseline.py); the operators never call them.
 """
 _OPS = ("gather", "scatter", "sort", "bincount_cumsum", "index_select_out", "batch_mm", "experts", "experts_backward",
         "router_topk", "router_topk_backward")
 _LAYERS = ("Yamoe", "experts_autograd")
+_BASELINES = {"reference": ".reference", "vendored": ".vendored", "yamoe_ref": ".vendored.yamoe_ref",
+              "gpt_oss_mlp": ".vendored.gpt_oss_mlp"}
 
-__all__ = ["ops", *_LAYERS, *_OPS]
+__all__ = ["ops", *_LAYERS, *_OPS, *_BASELINES]
 
 
 def __getattr__(name):
@@ -22,6 +26,10 @@ def __getattr__(name):
         from . import layers
 
         value = getattr(layers, name)
+    elif name in _BASELINES:
+        import importlib
+
+        value = importlib.import_module(_BASELINES[name], __name__)
     else:
         raise AttributeError("module %r has no attribute %r" % (__name__, name))
     globals()[name] = value
