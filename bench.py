@@ -260,6 +260,25 @@ def main():
                                    against="fp32 autograd through the oracle, all six gradients (worst shown)")
             del grads, want
         configs["cfg5_gptoss20b_backward_bf16"] = entry
+
+        # a training step of the layer: forward + backward.  With the reference's interface the backward recomputes the
+        # first product (experts + experts_backward); the pair experts_keep / experts_backward_kept hands the forward's
+        # activations over instead (T*K*3*I values of memory).
+        def step_recompute():
+            yamoe_amd.experts(*a, T, E, K)
+            yamoe_amd.experts_backward(gy, *a, T, E, K)
+
+        def step_kept():
+            _, kept = yamoe_amd.experts_keep(*a, T, E, K)
+            yamoe_amd.experts_backward_kept(gy, *a, kept, T, E, K)
+
+        ms_re, ms_kept = timed(step_recompute, few), timed(step_kept, few)
+        ms_bk = timed(lambda kept=yamoe_amd.experts_keep(*a, T, E, K)[1]: yamoe_amd.experts_backward_kept(gy, *a, kept, T, E, K), few)
+        configs["train_step_gptoss20b_bf16"] = dict(
+            ms_forward_plus_backward=round(ms_re, 4), ms_with_kept_activations=round(ms_kept, 4),
+            ms_backward_kept_alone=round(ms_bk, 4), kept_bytes=int(n_rows * 3 * I * 2),
+            note="forward + backward of one layer call; 'kept' = experts_keep + experts_backward_kept (no recomputation of "
+                 "the gate_up product in the backward)")
         del gy
     del d, a, hs
     torch.cuda.empty_cache()

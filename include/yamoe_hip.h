@@ -25,7 +25,9 @@ extern "C" {
 
 /* 2: YAMOE_F64 dtype code; yamoe_experts_forward_static; yamoe_route_workspace_bytes returns the size of a
  *    segments x buckets table above 4096 assignments (it was a constant 256 bytes); stream_max_rows up to 32;
- *    yamoe_probe_mfma_rate; yamoe_router_topk takes fp32; yamoe_router_backward; the whole op takes YAMOE_F64. */
+ *    yamoe_probe_mfma_rate; yamoe_router_topk takes fp32; yamoe_router_backward; the whole op takes YAMOE_F64.
+ *    Added since, without a change of existing behaviour: yamoe_experts_kept_bytes / _forward_keep / _backward_kept;
+ *    stream_max_rows = -1; H and I of any size; hidden_states of 4 GiB or more. */
 #define YAMOE_ABI_VERSION 2
 
 /* element type of activations, weights, biases and routing weights.  YAMOE_F64 is taken by the whole forward and
@@ -173,6 +175,30 @@ int yamoe_experts_backward(const yamoe_problem *p, const void *grad_out,
                            void *d_gate_up_proj, void *d_gate_up_proj_bias, void *d_down_proj,
                            void *d_down_proj_bias, void *workspace, size_t workspace_bytes,
                            void *stream);
+
+/* ---- the training pair: a forward that keeps what the backward would recompute ----
+ * No counterpart in the reference, whose backward recomputes the first product from hidden_states
+ * (csrc/experts_backward.cu:164-230); for callers that run the backward of the same call and can spare
+ * the memory (torch autograd with save_activations, a training loop).  yamoe_experts_forward_keep is
+ * yamoe_experts_forward that also leaves the activations [T*K, I] and the pre-activations [T*K, 2I] (sorted-row
+ * order, activation dtype) in `kept` (yamoe_experts_kept_bytes(p) bytes); yamoe_experts_backward_kept is
+ * yamoe_experts_backward on the same problem and inputs that reads them instead of running the gate_up
+ * product again (4*H*I of its 16*H*I flop per assignment).  Same workspaces, same outputs; experts that the
+ * forward served from its weight-streaming kernel differ from a recomputation in the last bits of their rows. */
+size_t yamoe_experts_kept_bytes(const yamoe_problem *p);
+int yamoe_experts_forward_keep(const yamoe_problem *p, const void *hidden_states,
+                               const void *router_indices, const void *routing_weights,
+                               const void *gate_up_proj, const void *gate_up_proj_bias,
+                               const void *down_proj, const void *down_proj_bias, void *out,
+                               void *kept, size_t kept_bytes, void *workspace, size_t workspace_bytes,
+                               void *stream);
+int yamoe_experts_backward_kept(const yamoe_problem *p, const void *grad_out, const void *hidden_states,
+                                const void *router_indices, const void *routing_weights,
+                                const void *gate_up_proj, const void *gate_up_proj_bias,
+                                const void *down_proj, const void *down_proj_bias, const void *kept,
+                                size_t kept_bytes, void *d_hidden, void *d_routing, void *d_gate_up_proj,
+                                void *d_gate_up_proj_bias, void *d_down_proj, void *d_down_proj_bias,
+                                void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- helper ops on the reference's own layouts (torch-ext/torch_binding.cpp:9-56) ---------
  * These serve code written against the reference's public helper ops; the fused forward and

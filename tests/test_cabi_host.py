@@ -170,3 +170,19 @@ def test_operators_answer_shape_queries_without_a_gpu():
     assert indices.shape == (T, K) and indices.dtype == torch.int64 and scores.shape == (T, E)
     d_hidden, d_weight, d_bias = yamoe_amd.router_topk_backward(scores, indices, scores, x, m(E, H))
     assert d_hidden.shape == (T, H) and d_weight.shape == (E, H) and d_bias.shape == (E,)
+
+
+def test_kept_bytes_matches_the_shape_function():
+    """yamoe_experts_kept_bytes (the buffer `experts_keep` returns) against the size the operator's shape function
+    reports to a graph capture."""
+    import yamoe_amd
+    from yamoe_amd import _cabi
+    lib = _cabi.lib()
+    for T, K, E, H, I, dt, code in ((12, 2, 4, 64, 48, torch.bfloat16, _cabi.BF16), (4096, 4, 32, 2880, 2880, torch.bfloat16, _cabi.BF16),
+                                    (7, 3, 5, 40, 33, torch.float32, _cabi.F32), (9, 1, 2, 8, 5, torch.float64, _cabi.F64)):
+        p = _cabi.Problem(T=T, K=K, E=E, H=H, I=I, capacity=T, dtype=code, idx_i64=1, rw_cols=E)
+        m = lambda *shape, dtype=dt: torch.empty(*shape, dtype=dtype, device="meta")
+        out, kept = yamoe_amd.experts_keep(m(T, H), m(T, K, dtype=torch.int64), m(T, E), m(E, H, 2 * I), m(E, 2 * I),
+                                           m(E, I, H), m(E, H), T, E, K)
+        assert out.shape == (T, H) and kept.dtype == torch.uint8
+        assert kept.numel() == lib.yamoe_experts_kept_bytes(ctypes.byref(p)), (T, K, I)

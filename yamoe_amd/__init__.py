@@ -7,7 +7,7 @@ the C ABI of libyamoe_hip.so; the first use of any of them fails if the native l
 to compare against (torch_baseline.py); the operators never call them.
 """
 _OPS = ("gather", "scatter", "sort", "bincount_cumsum", "index_select_out", "batch_mm", "experts", "experts_backward",
-        "router_topk", "router_topk_backward")
+        "router_topk", "router_topk_backward", "experts_keep", "experts_backward_kept")
 _LAYERS = ("Yamoe", "experts_autograd")
 _BASELINES = {"reference": ".reference", "vendored": ".vendored", "yamoe_ref": ".vendored.yamoe_ref",
               "gpt_oss_mlp": ".vendored.gpt_oss_mlp"}

@@ -26,6 +26,7 @@ SYMBOLS = [
     "yamoe_padded_scatter_workspace_bytes", "yamoe_padded_scatter", "yamoe_index_select", "yamoe_regular_groups",
     "yamoe_batch_mm_workspace_bytes", "yamoe_batch_mm", "yamoe_router_topk", "yamoe_probe_mfma_rate",
     "yamoe_router_backward_workspace_bytes", "yamoe_router_backward",
+    "yamoe_experts_kept_bytes", "yamoe_experts_forward_keep", "yamoe_experts_backward_kept",
 ]
 
 
@@ -66,6 +67,10 @@ def lib():
         L.yamoe_experts_backward_workspace_bytes.restype = sz
         L.yamoe_experts_backward_workspace_bytes.argtypes = [pp]
         L.yamoe_experts_backward.argtypes = [pp] + [vp] * 15 + [sz, vp]
+        L.yamoe_experts_kept_bytes.restype = sz
+        L.yamoe_experts_kept_bytes.argtypes = [pp]
+        L.yamoe_experts_forward_keep.argtypes = [pp] + [vp] * 8 + [vp, sz, vp, sz, vp]
+        L.yamoe_experts_backward_kept.argtypes = [pp] + [vp] * 8 + [vp, sz] + [vp] * 6 + [vp, sz, vp]
         L.yamoe_router_topk.argtypes = [vp, vp, vp, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp]
         L.yamoe_router_backward_workspace_bytes.restype = sz
         L.yamoe_router_backward_workspace_bytes.argtypes = [i32, i32, i32]

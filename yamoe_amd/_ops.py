@@ -21,7 +21,7 @@ for _p in (_LIB_HIP, _LIB_OPS):
 torch.ops.load_library(_LIB_OPS)
 ops = torch.ops._yamoe_amd_ops
 for _name in ("experts", "experts_backward", "gather", "scatter", "sort", "bincount_cumsum", "index_select_out", "batch_mm",
-              "router_topk", "router_topk_backward"):
+              "router_topk", "router_topk_backward", "experts_keep", "experts_backward_kept"):
     if not hasattr(ops, _name):
         raise ImportError("%s is stale (no operator %r): rebuild with `python -m yamoe_amd.build`" % (_LIB_OPS, _name))
 
@@ -43,6 +43,24 @@ def _register_fakes():
     @fake("_yamoe_amd_ops::experts_backward")
     def _(grad_out, hidden_states, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
           down_proj_bias, expert_capacity, num_experts, top_k):
+        return [t.new_empty(t.shape) for t in (hidden_states, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
+                                               down_proj_bias)]
+
+    def kept_bytes(hidden_states, router_indices, gate_up_proj):
+        # act [N, I] + pre [N, 2I], each region rounded up to 256 bytes (yamoe_experts_kept_bytes)
+        n, i, es = router_indices.shape[0] * router_indices.shape[1], gate_up_proj.shape[2] // 2, hidden_states.element_size()
+        up = lambda b: (max(b, 1) + 255) // 256 * 256
+        return up(n * i * es) + up(n * 2 * i * es)
+
+    @fake("_yamoe_amd_ops::experts_keep")
+    def _(hidden_states, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj, down_proj_bias,
+          expert_capacity, num_experts, top_k):
+        return (hidden_states.new_empty(hidden_states.shape),
+                hidden_states.new_empty((kept_bytes(hidden_states, router_indices, gate_up_proj),), dtype=torch.uint8))
+
+    @fake("_yamoe_amd_ops::experts_backward_kept")
+    def _(grad_out, hidden_states, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
+          down_proj_bias, kept, expert_capacity, num_experts, top_k):
         return [t.new_empty(t.shape) for t in (hidden_states, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
                                                down_proj_bias)]
 

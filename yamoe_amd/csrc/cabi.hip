@@ -103,12 +103,13 @@ int launch_router_backward_logits(const void *, const long long *, const void *,
 // the plain-FMA path (plain.hip): double precision, and sizes that are not whole 16-byte chunks
 template <typename T>
 int plain_forward(const void *, const void *, int, const void *, int, const void *, const void *, const void *, const void *,
-                  void *, const int *, const int *, const void *, void *, void *, int, int, int, int, int, hipStream_t);
+                  void *, const int *, const int *, const void *, void *, void *, void *, int, int, int, int, int,
+                  hipStream_t);
 template <typename T>
 int plain_backward(const void *, const void *, const void *, int, const void *, int, const void *, const void *, const void *,
                    const void *, void *, void *, void *, void *, void *, void *, const int *, const int *, const int *,
                    const int *, const int *, const void *, void *, void *, void *, void *, void *, void *, void *, void *, int,
-                   int, int, int, int, int, hipStream_t);
+                   int, int, int, int, int, int, hipStream_t);
 template <typename T> int plain_fill_zero(void *, long long, hipStream_t);
 
 template <typename T> struct HasStreamPath { static constexpr bool value = sizeof(T) == 2; };
@@ -311,6 +312,19 @@ static size_t carve_backward(const yamoe_problem *p, void *ws, BackwardBuffers *
   return used + c.used;
 }
 
+// What a forward can keep for the backward of the same call: the activations [N, I] and the pre-activations [N, 2I]
+// in sorted-row order (the backward otherwise recomputes both: the gate_up product once more).
+struct Saved {
+  void *act, *pre;
+};
+static size_t carve_saved(const yamoe_problem *p, void *base, Saved *s) {
+  const size_t N = (size_t)p->T * p->K, es = dtype_size(p->dtype);
+  Carver c(base);
+  s->act = c.take(N * p->I * es);
+  s->pre = c.take(N * 2 * p->I * es);
+  return c.used;
+}
+
 #define YAMOE_TRY(expr)        \
   do {                         \
     int rc_ = (expr);          \
@@ -319,9 +333,12 @@ static size_t carve_backward(const yamoe_problem *p, void *ws, BackwardBuffers *
 
 template <typename T>
 static int forward_impl(const yamoe_problem *p, const void *x, const void *idx, const void *rw, const void *wgu,
-                        const void *bgu, const void *wd, const void *bd, void *out, void *ws, hipStream_t stream) {
+                        const void *bgu, const void *wd, const void *bd, void *out, void *ws, const Saved *keep,
+                        hipStream_t stream) {
   ForwardBuffers b;
   carve_forward(p, ws, &b);
+  void *pre = nullptr;
+  if (keep != nullptr) { b.act = keep->act; pre = keep->pre; }  // (the workspace's own act region is then unused)
   const int N = p->T * p->K;
   void *st = (void *)stream;
   if (N == 0 || p->T == 0) return 0;
@@ -337,14 +354,14 @@ static int forward_impl(const yamoe_problem *p, const void *x, const void *idx, 
   const bool tiles = !everything && N > stream_rows;
   if (tiles && b.x_perm != nullptr) {  // (a hidden_states tensor too large to gather from: see gathers_need_permute)
     YAMOE_TRY(launch_permute<T>(x, b.sorted_idx, b.x_perm, N, p->K, p->H, stream));
-    YAMOE_TRY(tiles_gate_up<T>(b.x_perm, nullptr, wgu, bgu, b.act, nullptr, b.schedule, N, p->K, p->E, p->H, p->I, stream_rows,
+    YAMOE_TRY(tiles_gate_up<T>(b.x_perm, nullptr, wgu, bgu, b.act, pre, b.schedule, N, p->K, p->E, p->H, p->I, stream_rows,
                                stream));
   } else if (tiles) {
-    YAMOE_TRY(tiles_gate_up<T>(x, b.sorted_idx, wgu, bgu, b.act, nullptr, b.schedule, N, p->K, p->E, p->H, p->I, stream_rows,
+    YAMOE_TRY(tiles_gate_up<T>(x, b.sorted_idx, wgu, bgu, b.act, pre, b.schedule, N, p->K, p->E, p->H, p->I, stream_rows,
                                stream));
   }
   if constexpr (HasStreamPath<T>::value)
-    YAMOE_TRY(stream_gate_up<T>(x, b.sorted_idx, wgu, bgu, b.act, nullptr, b.schedule, N, p->K, p->E, p->H, p->I,
+    YAMOE_TRY(stream_gate_up<T>(x, b.sorted_idx, wgu, bgu, b.act, pre, b.schedule, N, p->K, p->E, p->H, p->I,
                                 stream));
   if (tiles) YAMOE_TRY(tiles_down<T>(b.act, wd, bd, b.y_perm, b.schedule, N, p->E, p->H, p->I, stream_rows, stream));
   if constexpr (HasStreamPath<T>::value)
@@ -357,9 +374,11 @@ static int forward_impl(const yamoe_problem *p, const void *x, const void *idx, 
 template <typename T>
 static int backward_impl(const yamoe_problem *p, const void *gy, const void *x, const void *idx, const void *rw,
                          const void *wgu, const void *bgu, const void *wd, const void *bd, void *d_x, void *d_rw,
-                         void *d_wgu, void *d_bgu, void *d_wd, void *d_bd, void *ws, hipStream_t stream) {
+                         void *d_wgu, void *d_bgu, void *d_wd, void *d_bd, void *ws, const Saved *kept,
+                         hipStream_t stream) {
   BackwardBuffers b;
   carve_backward(p, ws, &b);
+  if (kept != nullptr) { b.f.act = kept->act; b.pre = kept->pre; }  // the forward's own: nothing to recompute
   const int N = p->T * p->K, E = p->E, H = p->H, I = p->I, cap = p->capacity < 0 ? 0 : p->capacity;
   const size_t es = sizeof(T);
   void *st = (void *)stream;
@@ -377,10 +396,13 @@ static int backward_impl(const yamoe_problem *p, const void *gy, const void *x, 
   const bool permuted = b.gy_perm != nullptr;  // hidden_states and grad_out too large to gather from
   const bool gathers = !permuted && wgrad_gathers<T>(H, 2 * I);
   if (!gathers) YAMOE_TRY(launch_permute<T>(x, b.f.sorted_idx, b.x_perm, N, p->K, H, stream));
-  if (permuted)
+  if (kept != nullptr) {
+    // activations and pre-activations come from the forward
+  } else if (permuted) {
     YAMOE_TRY(tiles_gate_up<T>(b.x_perm, nullptr, wgu, bgu, b.f.act, b.pre, b.f.schedule, N, p->K, E, H, I, 0, stream));
-  else
+  } else {
     YAMOE_TRY(tiles_gate_up<T>(x, b.f.sorted_idx, wgu, bgu, b.f.act, b.pre, b.f.schedule, N, p->K, E, H, I, 0, stream));
+  }
   // combine backward: g_y_perm = grad_out[tok] * w, and the bias part of the routing gradient
   YAMOE_TRY(launch_combine_backward<T>(gy, bd, b.f.sorted_idx, b.f.inv_pos, idx, p->idx_i64, rw, p->rw_cols, b.g_y_perm,
                                        b.w_sorted, b.row_dot, N, p->K, E, H, stream));
@@ -431,23 +453,25 @@ static bool takes_plain_path(const yamoe_problem *p) {
 
 template <typename T>
 static int forward_plain(const yamoe_problem *p, const void *x, const void *idx, const void *rw, const void *wgu,
-                       const void *bgu, const void *wd, const void *bd, void *out, void *ws, hipStream_t stream) {
+                       const void *bgu, const void *wd, const void *bd, void *out, void *ws, const Saved *keep,
+                       hipStream_t stream) {
   ForwardBuffers b;
   carve_forward(p, ws, &b);
   const int N = p->T * p->K;
   if (N == 0 || p->T == 0) return 0;
   YAMOE_TRY(route_and_schedule(idx, p->idx_i64, N, p->E, p->capacity, b.sorted_expert, b.sorted_idx, b.counts, b.offsets,
                                b.inv_pos, b.route_ws, b.route_ws_bytes, 0, b.schedule, b.schedule_bytes, (void *)stream));
-  return plain_forward<T>(x, idx, p->idx_i64, rw, p->rw_cols, wgu, bgu, wd, bd, out, b.sorted_idx, b.inv_pos, b.schedule, b.act,
-                     b.y_perm, p->T, p->K, p->E, p->H, p->I, stream);
+  return plain_forward<T>(x, idx, p->idx_i64, rw, p->rw_cols, wgu, bgu, wd, bd, out, b.sorted_idx, b.inv_pos, b.schedule,
+                          keep ? keep->act : b.act, keep ? keep->pre : nullptr, b.y_perm, p->T, p->K, p->E, p->H, p->I, stream);
 }
 
 template <typename T>
 static int backward_plain(const yamoe_problem *p, const void *gy, const void *x, const void *idx, const void *rw,
                         const void *wgu, const void *bgu, const void *wd, const void *bd, void *d_x, void *d_rw, void *d_wgu,
-                        void *d_bgu, void *d_wd, void *d_bd, void *ws, hipStream_t stream) {
+                        void *d_bgu, void *d_wd, void *d_bd, void *ws, const Saved *kept, hipStream_t stream) {
   BackwardBuffers b;
   carve_backward(p, ws, &b);
+  if (kept != nullptr) { b.f.act = kept->act; b.pre = kept->pre; }
   const int N = p->T * p->K, E = p->E, H = p->H, I = p->I, cap = p->capacity < 0 ? 0 : p->capacity;
   if (N == 0) {
     YAMOE_TRY(plain_fill_zero<T>(d_rw, (long long)p->T * p->rw_cols, stream));
@@ -462,7 +486,8 @@ static int backward_plain(const yamoe_problem *p, const void *gy, const void *x,
                                (void *)stream));
   return plain_backward<T>(gy, x, idx, p->idx_i64, rw, p->rw_cols, wgu, bgu, wd, bd, d_x, d_rw, d_wgu, d_bgu, d_wd, d_bd,
                       b.f.sorted_expert, b.f.sorted_idx, b.f.inv_pos, b.f.counts, b.f.offsets, b.f.schedule, b.f.act, b.pre,
-                      b.g_y_perm, b.d_act, b.d_pre, b.d_x_perm, b.w_sorted, b.row_dot, p->T, p->K, E, H, I, cap, stream);
+                      b.g_y_perm, b.d_act, b.d_pre, b.d_x_perm, b.w_sorted, b.row_dot, p->T, p->K, E, H, I, cap,
+                      kept == nullptr ? 1 : 0, stream);
 }
 
 }  // namespace yamoe
@@ -555,30 +580,62 @@ extern "C" size_t yamoe_experts_workspace_bytes(const yamoe_problem *p) {
   return carve_forward(p, nullptr, &b);
 }
 
-extern "C" int yamoe_experts_forward(const yamoe_problem *p, const void *hidden_states, const void *router_indices,
-                                     const void *routing_weights, const void *gate_up_proj,
-                                     const void *gate_up_proj_bias, const void *down_proj, const void *down_proj_bias,
-                                     void *out, void *workspace, size_t workspace_bytes, void *stream) {
-  YAMOE_TRY(check_problem(p, "yamoe_experts_forward"));
+// checks and dispatch shared by yamoe_experts_forward and yamoe_experts_forward_keep
+static int run_forward(const char *who, const yamoe_problem *p, const void *hidden_states, const void *router_indices,
+                       const void *routing_weights, const void *gate_up_proj, const void *gate_up_proj_bias,
+                       const void *down_proj, const void *down_proj_bias, void *out, void *kept, size_t kept_bytes,
+                       bool keeps, void *workspace, size_t workspace_bytes, void *stream) {
+  YAMOE_TRY(check_problem(p, who));
   if (p->T == 0) return 0;
   if (!hidden_states || !router_indices || !routing_weights || !gate_up_proj || !gate_up_proj_bias || !down_proj ||
-      !down_proj_bias || !out || !workspace) {
-    set_error("yamoe_experts_forward: null pointer");
+      !down_proj_bias || !out || !workspace || (keeps && !kept)) {
+    set_error("%s: null pointer", who);
     return YAMOE_E_ARG;
   }
   size_t need = yamoe_experts_workspace_bytes(p);
   if (workspace_bytes < need) {
-    set_error("yamoe_experts_forward: workspace too small (%zu < %zu)", workspace_bytes, need);
+    set_error("%s: workspace too small (%zu < %zu)", who, workspace_bytes, need);
     return YAMOE_E_WORKSPACE;
   }
+  Saved sv = {};
+  if (keeps && kept_bytes < carve_saved(p, kept, &sv)) {
+    set_error("%s: the buffer for the kept activations is too small (%zu < %zu)", who, kept_bytes, carve_saved(p, nullptr, &sv));
+    return YAMOE_E_WORKSPACE;
+  }
+  const Saved *keep = keeps ? &sv : nullptr;
   if (takes_plain_path(p)) {
     YAMOE_DISPATCH_ALL(p->dtype, forward_plain<T>(p, hidden_states, router_indices, routing_weights, gate_up_proj,
-                                                  gate_up_proj_bias, down_proj, down_proj_bias, out, workspace,
+                                                  gate_up_proj_bias, down_proj, down_proj_bias, out, workspace, keep,
                                                   (hipStream_t)stream));
   }
   YAMOE_DISPATCH(p->dtype, forward_impl<T>(p, hidden_states, router_indices, routing_weights, gate_up_proj,
-                                           gate_up_proj_bias, down_proj, down_proj_bias, out, workspace,
+                                           gate_up_proj_bias, down_proj, down_proj_bias, out, workspace, keep,
                                            (hipStream_t)stream));
+}
+
+extern "C" int yamoe_experts_forward(const yamoe_problem *p, const void *hidden_states, const void *router_indices,
+                                     const void *routing_weights, const void *gate_up_proj,
+                                     const void *gate_up_proj_bias, const void *down_proj, const void *down_proj_bias,
+                                     void *out, void *workspace, size_t workspace_bytes, void *stream) {
+  return run_forward("yamoe_experts_forward", p, hidden_states, router_indices, routing_weights, gate_up_proj,
+                     gate_up_proj_bias, down_proj, down_proj_bias, out, nullptr, 0, false, workspace, workspace_bytes, stream);
+}
+
+// ---- the training pair: a forward that keeps what the backward would recompute ----------------------------------
+extern "C" size_t yamoe_experts_kept_bytes(const yamoe_problem *p) {
+  if (check_problem(p, "yamoe_experts_kept_bytes")) return 0;
+  Saved sv;
+  return carve_saved(p, nullptr, &sv);
+}
+
+extern "C" int yamoe_experts_forward_keep(const yamoe_problem *p, const void *hidden_states, const void *router_indices,
+                                          const void *routing_weights, const void *gate_up_proj,
+                                          const void *gate_up_proj_bias, const void *down_proj,
+                                          const void *down_proj_bias, void *out, void *kept, size_t kept_bytes,
+                                          void *workspace, size_t workspace_bytes, void *stream) {
+  return run_forward("yamoe_experts_forward_keep", p, hidden_states, router_indices, routing_weights, gate_up_proj,
+                     gate_up_proj_bias, down_proj, down_proj_bias, out, kept, kept_bytes, true, workspace, workspace_bytes,
+                     stream);
 }
 
 // ---- the forward without a workspace argument ----------------------------------------------------------
@@ -633,11 +690,12 @@ extern "C" int yamoe_experts_forward_static(const yamoe_problem *p, const void *
   // in the same call, so the contents left by the previous call on this GPU do not matter.
   if (takes_plain_path(p)) {
     YAMOE_DISPATCH_ALL(p->dtype, forward_plain<T>(p, hidden_states, router_indices, routing_weights, gate_up_proj,
-                                                  gate_up_proj_bias, down_proj, down_proj_bias, out, ws,
+                                                  gate_up_proj_bias, down_proj, down_proj_bias, out, ws, nullptr,
                                                   (hipStream_t)stream));
   }
   YAMOE_DISPATCH(p->dtype, forward_impl<T>(p, hidden_states, router_indices, routing_weights, gate_up_proj,
-                                           gate_up_proj_bias, down_proj, down_proj_bias, out, ws, (hipStream_t)stream));
+                                           gate_up_proj_bias, down_proj, down_proj_bias, out, ws, nullptr,
+                                           (hipStream_t)stream));
 }
 
 extern "C" size_t yamoe_experts_backward_workspace_bytes(const yamoe_problem *p) {
@@ -646,34 +704,64 @@ extern "C" size_t yamoe_experts_backward_workspace_bytes(const yamoe_problem *p)
   return carve_backward(p, nullptr, &b);
 }
 
+static int run_backward(const char *who, const yamoe_problem *p, const void *grad_out, const void *hidden_states,
+                        const void *router_indices, const void *routing_weights, const void *gate_up_proj,
+                        const void *gate_up_proj_bias, const void *down_proj, const void *down_proj_bias,
+                        const void *kept, size_t kept_bytes, bool has_kept, void *d_hidden, void *d_routing,
+                        void *d_gate_up_proj, void *d_gate_up_proj_bias, void *d_down_proj, void *d_down_proj_bias,
+                        void *workspace, size_t workspace_bytes, void *stream) {
+  YAMOE_TRY(check_problem(p, who));
+  if (!gate_up_proj || !gate_up_proj_bias || !down_proj || !down_proj_bias || !d_gate_up_proj ||
+      !d_gate_up_proj_bias || !d_down_proj || !d_down_proj_bias || !workspace ||
+      (p->T > 0 && (!grad_out || !hidden_states || !router_indices || !routing_weights || !d_hidden || !d_routing ||
+                    (has_kept && !kept)))) {
+    set_error("%s: null pointer", who);
+    return YAMOE_E_ARG;
+  }
+  size_t need = yamoe_experts_backward_workspace_bytes(p);
+  if (workspace_bytes < need) {
+    set_error("%s: workspace too small (%zu < %zu)", who, workspace_bytes, need);
+    return YAMOE_E_WORKSPACE;
+  }
+  Saved sv = {};
+  if (has_kept && kept_bytes < carve_saved(p, (void *)kept, &sv)) {
+    set_error("%s: the buffer of kept activations is too small (%zu < %zu)", who, kept_bytes, carve_saved(p, nullptr, &sv));
+    return YAMOE_E_WORKSPACE;
+  }
+  const Saved *k = has_kept && p->T > 0 ? &sv : nullptr;
+  if (takes_plain_path(p)) {
+    YAMOE_DISPATCH_ALL(p->dtype, backward_plain<T>(p, grad_out, hidden_states, router_indices, routing_weights, gate_up_proj,
+                                                   gate_up_proj_bias, down_proj, down_proj_bias, d_hidden, d_routing,
+                                                   d_gate_up_proj, d_gate_up_proj_bias, d_down_proj, d_down_proj_bias,
+                                                   workspace, k, (hipStream_t)stream));
+  }
+  YAMOE_DISPATCH(p->dtype, backward_impl<T>(p, grad_out, hidden_states, router_indices, routing_weights, gate_up_proj,
+                                            gate_up_proj_bias, down_proj, down_proj_bias, d_hidden, d_routing,
+                                            d_gate_up_proj, d_gate_up_proj_bias, d_down_proj, d_down_proj_bias,
+                                            workspace, k, (hipStream_t)stream));
+}
+
 extern "C" int yamoe_experts_backward(const yamoe_problem *p, const void *grad_out, const void *hidden_states,
                                       const void *router_indices, const void *routing_weights,
                                       const void *gate_up_proj, const void *gate_up_proj_bias, const void *down_proj,
                                       const void *down_proj_bias, void *d_hidden, void *d_routing,
                                       void *d_gate_up_proj, void *d_gate_up_proj_bias, void *d_down_proj,
                                       void *d_down_proj_bias, void *workspace, size_t workspace_bytes, void *stream) {
-  YAMOE_TRY(check_problem(p, "yamoe_experts_backward"));
-  if (!gate_up_proj || !gate_up_proj_bias || !down_proj || !down_proj_bias || !d_gate_up_proj ||
-      !d_gate_up_proj_bias || !d_down_proj || !d_down_proj_bias || !workspace ||
-      (p->T > 0 && (!grad_out || !hidden_states || !router_indices || !routing_weights || !d_hidden || !d_routing))) {
-    set_error("yamoe_experts_backward: null pointer");
-    return YAMOE_E_ARG;
-  }
-  size_t need = yamoe_experts_backward_workspace_bytes(p);
-  if (workspace_bytes < need) {
-    set_error("yamoe_experts_backward: workspace too small (%zu < %zu)", workspace_bytes, need);
-    return YAMOE_E_WORKSPACE;
-  }
-  if (takes_plain_path(p)) {
-    YAMOE_DISPATCH_ALL(p->dtype, backward_plain<T>(p, grad_out, hidden_states, router_indices, routing_weights, gate_up_proj,
-                                                   gate_up_proj_bias, down_proj, down_proj_bias, d_hidden, d_routing,
-                                                   d_gate_up_proj, d_gate_up_proj_bias, d_down_proj, d_down_proj_bias,
-                                                   workspace, (hipStream_t)stream));
-  }
-  YAMOE_DISPATCH(p->dtype, backward_impl<T>(p, grad_out, hidden_states, router_indices, routing_weights, gate_up_proj,
-                                            gate_up_proj_bias, down_proj, down_proj_bias, d_hidden, d_routing,
-                                            d_gate_up_proj, d_gate_up_proj_bias, d_down_proj, d_down_proj_bias,
-                                            workspace, (hipStream_t)stream));
+  return run_backward("yamoe_experts_backward", p, grad_out, hidden_states, router_indices, routing_weights, gate_up_proj,
+                      gate_up_proj_bias, down_proj, down_proj_bias, nullptr, 0, false, d_hidden, d_routing, d_gate_up_proj,
+                      d_gate_up_proj_bias, d_down_proj, d_down_proj_bias, workspace, workspace_bytes, stream);
+}
+
+extern "C" int yamoe_experts_backward_kept(const yamoe_problem *p, const void *grad_out, const void *hidden_states,
+                                           const void *router_indices, const void *routing_weights,
+                                           const void *gate_up_proj, const void *gate_up_proj_bias,
+                                           const void *down_proj, const void *down_proj_bias, const void *kept,
+                                           size_t kept_bytes, void *d_hidden, void *d_routing, void *d_gate_up_proj,
+                                           void *d_gate_up_proj_bias, void *d_down_proj, void *d_down_proj_bias,
+                                           void *workspace, size_t workspace_bytes, void *stream) {
+  return run_backward("yamoe_experts_backward_kept", p, grad_out, hidden_states, router_indices, routing_weights,
+                      gate_up_proj, gate_up_proj_bias, down_proj, down_proj_bias, kept, kept_bytes, true, d_hidden, d_routing,
+                      d_gate_up_proj, d_gate_up_proj_bias, d_down_proj, d_down_proj_bias, workspace, workspace_bytes, stream);
 }
 
 // ---- gradient of the router step ------------------------------------------------------------------------

@@ -343,14 +343,15 @@ static int plain_gate_up_down(const T *x, const int *sorted_idx, const T *wgu, c
   return 0;
 }
 
-// The whole forward on the caller's lists (sorted_idx, inv_pos, schedule built with no streaming limit).
+// The whole forward on the caller's lists (sorted_idx, inv_pos, schedule built with no streaming limit); `pre` (optional)
+// receives the pre-activations.
 template <typename T>
 int plain_forward(const void *x, const void *idx, int idx_i64, const void *rw, int rw_cols, const void *wgu, const void *bgu,
                   const void *wd, const void *bd, void *out, const int *sorted_idx, const int *inv_pos, const void *sched,
-                  void *act, void *y_perm, int Tn, int K, int E, int H, int I, hipStream_t stream) {
+                  void *act, void *pre, void *y_perm, int Tn, int K, int E, int H, int I, hipStream_t stream) {
   const int N = Tn * K;
   PLAIN_TRY(plain_gate_up_down<T>((const T *)x, sorted_idx, (const T *)wgu, (const T *)bgu, (const T *)wd, (const T *)bd,
-                                  (T *)act, nullptr, (T *)y_perm, sched, N, K, E, H, I, stream));
+                                  (T *)act, (T *)pre, (T *)y_perm, sched, N, K, E, H, I, stream));
   hipLaunchKernelGGL(plain::combine_kernel<T>, dim3(Tn), dim3(256), 0, stream, (const T *)y_perm, inv_pos, idx, idx_i64,
                      (const T *)rw, rw_cols, (T *)out, Tn, K, E, H);
   return check_launch("plain combine_kernel");
@@ -364,7 +365,7 @@ int plain_backward(const void *gy_, const void *x_, const void *idx, int idx_i64
                    void *d_bgu, void *d_wd, void *d_bd, const int *sorted_expert, const int *sorted_idx, const int *inv_pos,
                    const int *counts, const int *offsets, const void *sched, void *act_, void *pre_, void *g_y_,
                    void *d_act_, void *d_pre_, void *d_x_perm_, void *w_sorted_, void *row_dot_, int Tn, int K, int E, int H,
-                   int I, int capacity, hipStream_t stream) {
+                   int I, int capacity, int recompute, hipStream_t stream) {
   typedef typename plain::AccOf<T>::type A;
   const int N = Tn * K;
   const T *gy = (const T *)gy_, *x = (const T *)x_, *rw = (const T *)rw_;
@@ -372,8 +373,8 @@ int plain_backward(const void *gy_, const void *x_, const void *idx, int idx_i64
   T *act = (T *)act_, *pre = (T *)pre_, *g_y = (T *)g_y_, *d_act = (T *)d_act_;
   T *d_pre = (T *)d_pre_, *d_x_perm = (T *)d_x_perm_;
   A *w_sorted = (A *)w_sorted_, *row_dot = (A *)row_dot_;
-  // forward recompute of the first product: activations and pre-activations
-  PLAIN_TRY(plain_gate_up_down<T>(x, sorted_idx, wgu, bgu, wd, bd, act, pre, nullptr, sched, N, K, E, H, I, stream));
+  // forward recompute of the first product: activations and pre-activations (unless the caller kept the forward's)
+  if (recompute) PLAIN_TRY(plain_gate_up_down<T>(x, sorted_idx, wgu, bgu, wd, bd, act, pre, nullptr, sched, N, K, E, H, I, stream));
   // weighted rows of grad_out; bias and weight gradient of the down projection
   hipLaunchKernelGGL(plain::scale_rows_kernel<T>, dim3(N), dim3(256), 0, stream, gy, sorted_idx, inv_pos, idx, idx_i64, rw,
                      rw_cols, g_y, w_sorted, N, K, E, H);
@@ -429,12 +430,12 @@ template <typename T> int plain_fill_zero(void *p, long long n, hipStream_t stre
 #define PLAIN_INSTANTIATE(T)                                                                                              \
   template int plain_forward<T>(const void *, const void *, int, const void *, int, const void *, const void *,          \
                                 const void *, const void *, void *, const int *, const int *, const void *, void *,      \
-                                void *, int, int, int, int, int, hipStream_t);                                            \
+                                void *, void *, int, int, int, int, int, hipStream_t);                                    \
   template int plain_backward<T>(const void *, const void *, const void *, int, const void *, int, const void *,         \
                                  const void *, const void *, const void *, void *, void *, void *, void *, void *,       \
                                  void *, const int *, const int *, const int *, const int *, const int *, const void *,  \
                                  void *, void *, void *, void *, void *, void *, void *, void *, int, int, int, int, int, \
-                                 int, hipStream_t);                                                                       \
+                                 int, int, hipStream_t);                                                                  \
   template int plain_fill_zero<T>(void *, long long, hipStream_t);
 PLAIN_INSTANTIATE(double)
 PLAIN_INSTANTIATE(float)

@@ -162,6 +162,66 @@ std::vector<at::Tensor> experts_backward(const at::Tensor &grad_out, const at::T
   return {d_hidden, d_routing, d_wgu, d_bgu, d_wd, d_bd};
 }
 
+// The training pair (no counterpart in the reference, which recomputes): `experts_keep` also returns the activations
+// and pre-activations as one byte tensor, `experts_backward_kept` takes it back in place of the recomputation.
+std::tuple<at::Tensor, at::Tensor> experts_keep(at::Tensor hidden_states, at::Tensor router_indices,
+                                                at::Tensor routing_weights, at::Tensor gate_up_proj,
+                                                at::Tensor gate_up_proj_bias, at::Tensor down_proj,
+                                                at::Tensor down_proj_bias, int64_t expert_capacity, int64_t num_experts,
+                                                int64_t top_k) {
+  Checked c = check_inputs(hidden_states, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
+                           down_proj_bias, expert_capacity, num_experts, top_k);
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(c.hidden.device());
+  at::Tensor out = at::empty_like(c.hidden);
+  const size_t kept_bytes = yamoe_experts_kept_bytes(&c.p);
+  at::Tensor kept = at::empty({(int64_t)kept_bytes}, c.hidden.options().dtype(at::kByte));
+  if (c.p.T == 0) return std::make_tuple(out, kept);
+  size_t ws_bytes = yamoe_experts_workspace_bytes(&c.p);
+  TORCH_CHECK(ws_bytes > 0, "experts_keep: ", yamoe_last_error());
+  at::Tensor ws = at::empty({(int64_t)ws_bytes}, c.hidden.options().dtype(at::kByte));
+  void *stream = (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+  check_rc(yamoe_experts_forward_keep(&c.p, c.hidden.data_ptr(), c.idx.data_ptr(), c.rw.data_ptr(), c.wgu.data_ptr(),
+                                      c.bgu.data_ptr(), c.wd.data_ptr(), c.bd.data_ptr(), out.data_ptr(), kept.data_ptr(),
+                                      kept_bytes, ws.data_ptr(), ws_bytes, stream),
+           "yamoe_experts_forward_keep");
+  return std::make_tuple(out, kept);
+}
+
+std::vector<at::Tensor> experts_backward_kept(const at::Tensor &grad_out, const at::Tensor &hidden_states,
+                                              const at::Tensor &router_indices, const at::Tensor &routing_weights,
+                                              const at::Tensor &gate_up_proj, const at::Tensor &gate_up_proj_bias,
+                                              const at::Tensor &down_proj, const at::Tensor &down_proj_bias,
+                                              const at::Tensor &kept, int64_t expert_capacity, int64_t num_experts,
+                                              int64_t top_k) {
+  TORCH_CHECK(grad_out.is_cuda(), "grad_out must be on the GPU");
+  Checked c = check_inputs(hidden_states, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
+                           down_proj_bias, expert_capacity, num_experts, top_k);
+  const int64_t T = c.p.T, H = c.p.H;
+  TORCH_CHECK(grad_out.scalar_type() == c.hidden.scalar_type(), "grad_out must share hidden_states' dtype");
+  TORCH_CHECK(grad_out.numel() == T * H, "grad_out must be [T, H]");
+  TORCH_CHECK(kept.is_cuda() && kept.scalar_type() == at::kByte && kept.is_contiguous() &&
+                  (size_t)kept.numel() >= yamoe_experts_kept_bytes(&c.p),
+              "kept must be the byte tensor that experts_keep returned for the same problem");
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(c.hidden.device());
+  at::Tensor gy = grad_out.contiguous().view({T, H});
+  at::Tensor d_hidden = at::empty_like(c.hidden);
+  at::Tensor d_routing = at::empty_like(c.rw);
+  at::Tensor d_wgu = at::empty_like(c.wgu);
+  at::Tensor d_bgu = at::empty_like(c.bgu);
+  at::Tensor d_wd = at::empty_like(c.wd);
+  at::Tensor d_bd = at::empty_like(c.bd);
+  size_t ws_bytes = yamoe_experts_backward_workspace_bytes(&c.p);
+  TORCH_CHECK(ws_bytes > 0, "experts_backward_kept: ", yamoe_last_error());
+  at::Tensor ws = at::empty({(int64_t)ws_bytes}, c.hidden.options().dtype(at::kByte));
+  void *stream = (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+  check_rc(yamoe_experts_backward_kept(&c.p, gy.data_ptr(), c.hidden.data_ptr(), c.idx.data_ptr(), c.rw.data_ptr(),
+                                       c.wgu.data_ptr(), c.bgu.data_ptr(), c.wd.data_ptr(), c.bd.data_ptr(),
+                                       kept.data_ptr(), (size_t)kept.numel(), d_hidden.data_ptr(), d_routing.data_ptr(),
+                                       d_wgu.data_ptr(), d_bgu.data_ptr(), d_wd.data_ptr(), d_bd.data_ptr(), ws.data_ptr(),
+                                       ws_bytes, stream),
+           "yamoe_experts_backward_kept");
+  return {d_hidden, d_routing, d_wgu, d_bgu, d_wd, d_bd};
+}
 
 // ---- helper ops on the reference's layouts (torch-ext/torch_binding.cpp:9-56) -----------------------------
 void *current_stream() { return (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream(); }
@@ -381,4 +441,13 @@ TORCH_LIBRARY(_yamoe_amd_ops, ops) {
           "int num_experts, "
           "int top_k) -> Tensor[]");
   ops.impl("experts_backward", c10::DispatchKey::CUDA, &experts_backward);
+
+  ops.def("experts_keep(Tensor hidden_states, Tensor router_indices, Tensor routing_weights, Tensor gate_up_proj, "
+          "Tensor gate_up_proj_bias, Tensor down_proj, Tensor down_proj_bias, int expert_capacity, int num_experts, "
+          "int top_k) -> (Tensor, Tensor)");
+  ops.impl("experts_keep", c10::DispatchKey::CUDA, &experts_keep);
+  ops.def("experts_backward_kept(Tensor grad_out, Tensor hidden_states, Tensor router_indices, Tensor routing_weights, "
+          "Tensor gate_up_proj, Tensor gate_up_proj_bias, Tensor down_proj, Tensor down_proj_bias, Tensor kept, "
+          "int expert_capacity, int num_experts, int top_k) -> Tensor[]");
+  ops.impl("experts_backward_kept", c10::DispatchKey::CUDA, &experts_backward_kept);
 }

@@ -11,33 +11,45 @@ from ._ops import ops
 class _ExpertsFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, hidden_flat, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
-                down_proj_bias, expert_capacity, num_experts, top_k, enable_router_grads):
-        out = ops.experts(hidden_flat, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
-                          down_proj_bias, expert_capacity, num_experts, top_k)
+                down_proj_bias, expert_capacity, num_experts, top_k, enable_router_grads, save_activations=False):
+        a = (hidden_flat, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj, down_proj_bias)
+        if save_activations:
+            # keep the activations and pre-activations ([T*K, 3I] values) for the backward instead of letting it run
+            # the gate_up product again: a fifth of the backward's time for that much memory
+            out, kept = ops.experts_keep(*a, expert_capacity, num_experts, top_k)
+        else:
+            out, kept = ops.experts(*a, expert_capacity, num_experts, top_k), None
         ctx.expert_capacity = expert_capacity
         ctx.num_experts = num_experts
         ctx.top_k = top_k
         ctx.enable_router_grads = bool(enable_router_grads)
-        ctx.save_for_backward(hidden_flat, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias,
-                              down_proj, down_proj_bias)
+        ctx.save_activations = kept is not None
+        ctx.save_for_backward(*a, *([kept] if kept is not None else []))
         return out
 
     @staticmethod
     def backward(ctx, grad_output):
         saved = ctx.saved_tensors
-        d_hidden, d_routing, d_wgu, d_bgu, d_wd, d_bd = ops.experts_backward(
-            grad_output.contiguous(), *saved, ctx.expert_capacity, ctx.num_experts, ctx.top_k)
+        if ctx.save_activations:
+            grads = ops.experts_backward_kept(grad_output.contiguous(), *saved, ctx.expert_capacity, ctx.num_experts,
+                                              ctx.top_k)
+        else:
+            grads = ops.experts_backward(grad_output.contiguous(), *saved, ctx.expert_capacity, ctx.num_experts, ctx.top_k)
+        d_hidden, d_routing, d_wgu, d_bgu, d_wd, d_bd = grads
         if not ctx.enable_router_grads:
             d_routing = None
-        return d_hidden, None, d_routing, d_wgu, d_bgu, d_wd, d_bd, None, None, None, None
+        return d_hidden, None, d_routing, d_wgu, d_bgu, d_wd, d_bd, None, None, None, None, None
 
 
 def experts_autograd(hidden_flat, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
-                     down_proj_bias, expert_capacity, num_experts, top_k, enable_router_grads=True):
+                     down_proj_bias, expert_capacity, num_experts, top_k, enable_router_grads=True,
+                     save_activations=False):
     """Differentiable `experts`: gradients flow to hidden states, weights, biases and (optionally)
-    the routing weights."""
+    the routing weights.  `save_activations` keeps the first product's results of the forward for the backward
+    (T*K*3*I values of memory) instead of recomputing them there as the reference does
+    (csrc/experts_backward.cu:164-230)."""
     return _ExpertsFn.apply(hidden_flat, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj,
-                            down_proj_bias, expert_capacity, num_experts, top_k, enable_router_grads)
+                            down_proj_bias, expert_capacity, num_experts, top_k, enable_router_grads, save_activations)
 
 
 class _RouterFn(torch.autograd.Function):
@@ -144,7 +156,7 @@ class Yamoe(torch.nn.Module):
         if want_router_grads:
             out = experts_autograd(x_flat, router_indices, router_scores, gate_up, gate_up_bias,
                                    self.experts.down_proj, self.experts.down_proj_bias, capacity, num_experts, top_k,
-                                   True)
+                                   True, bool(getattr(self, "save_activations", False)))
         else:
             with torch.no_grad():
                 out = ops.experts(x_flat, router_indices, router_scores, gate_up, gate_up_bias,
