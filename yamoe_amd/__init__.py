@@ -9,10 +9,10 @@ to compare against (torch_baseline.py); the operators never call them.
 _OPS = ("gather", "scatter", "sort", "bincount_cumsum", "index_select_out", "batch_mm", "experts", "experts_backward",
         "router_topk", "router_topk_backward", "experts_keep", "experts_backward_kept")
 _LAYERS = ("Yamoe", "experts_autograd")
-_BASELINES = {"reference": ".reference", "vendored": ".vendored", "yamoe_ref": ".vendored.yamoe_ref",
+_TORCH_MODULES = {"reference": ".reference", "vendored": ".vendored", "yamoe_ref": ".vendored.yamoe_ref",
               "gpt_oss_mlp": ".vendored.gpt_oss_mlp"}
 
-__all__ = ["ops", *_LAYERS, *_OPS, *_BASELINES]
+__all__ = ["ops", *_LAYERS, *_OPS, *_TORCH_MODULES]
 
 
 def __getattr__(name):
@@ -26,10 +26,10 @@ def __getattr__(name):
         from . import layers
 
         value = getattr(layers, name)
-    elif name in _BASELINES:
+    elif name in _TORCH_MODULES:
         import importlib
 
-        value = importlib.import_module(_BASELINES[name], __name__)
+        value = importlib.import_module(_TORCH_MODULES[name], __name__)
     else:
         raise AttributeError("module %r has no attribute %r" % (__name__, name))
     globals()[name] = value
