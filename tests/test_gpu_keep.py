@@ -25,6 +25,7 @@ SHAPES = [
     (600, 128, 64, 4, 2, 37, 0.5, True),       # capacity drops assignments
     (40, 64, 64, 16, 1, 0, 0.0, False),        # every expert streams
     (300, 67, 35, 5, 3, 0, 0.0, True),         # odd sizes: the plain-FMA kernels
+    (3, 64, 320, 2, 1, 0, 0.0, False),         # a handful of rows: the weight-gradient kernel's last slab runs past them
 ]
 
 

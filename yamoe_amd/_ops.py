@@ -47,10 +47,10 @@ def _register_fakes():
                                                down_proj_bias)]
 
     def kept_bytes(hidden_states, router_indices, gate_up_proj):
-        # act [N, I] + pre [N, 2I], each region rounded up to 256 bytes (yamoe_experts_kept_bytes)
+        # act [N, I] + pre [N, 2I] + 32 rows of I as a pad, each region rounded up to 256 bytes (yamoe_experts_kept_bytes)
         n, i, es = router_indices.shape[0] * router_indices.shape[1], gate_up_proj.shape[2] // 2, hidden_states.element_size()
         up = lambda b: (max(b, 1) + 255) // 256 * 256
-        return up(n * i * es) + up(n * 2 * i * es)
+        return up(n * i * es) + up(n * 2 * i * es) + up(32 * i * es)
 
     @fake("_yamoe_amd_ops::experts_keep")
     def _(hidden_states, router_indices, routing_weights, gate_up_proj, gate_up_proj_bias, down_proj, down_proj_bias,

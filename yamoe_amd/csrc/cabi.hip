@@ -322,6 +322,9 @@ static size_t carve_saved(const yamoe_problem *p, void *base, Saved *s) {
   Carver c(base);
   s->act = c.take(N * p->I * es);
   s->pre = c.take(N * 2 * p->I * es);
+  // the weight-gradient kernel's copies of an expert's last, partial slab of rows run up to 32 rows past the end of
+  // the activations: into the pre-activations, and for a handful of rows beyond those, into this pad
+  c.take(32 * (size_t)p->I * es);
   return c.used;
 }
 
