@@ -1,11 +1,14 @@
 """Timing sweep of the `experts` op over the shapes drbh/yamoe plots (perf_plot.py:29-39: six layer shapes x seven
 batch sizes, fp16, routing from random logits), one JSON line per point instead of a figure.
 
-    python -m yamoe_amd.sweep [--configs 0,1,..] [--batches 1,2,4,..] [--iters 20] [--capacity seq|tokens]
+    python -m yamoe_amd.sweep [--configs 0,1,..] [--batches 1,2,4,..] [--iters 20] [--capacity seq|tokens] [--torch]
 
 `--capacity seq` passes `seq_len` as `expert_capacity` like the reference script does (perf_plot.py:118: assignments
 beyond that rank inside an expert are dropped); `tokens` (default) keeps every assignment.  TFLOP/s counts
-6 * hidden^2 flop per kept assignment.
+6 * hidden^2 flop per kept assignment.  `--torch` also times the plain-torch experts module on the same GPU and inputs
+(perf_plot.py:104-146 times `reference.GptOssExperts` in inference mode next to the kernel and plots the ratio): here
+`yamoe_amd.reference.GptOssExperts`, in its per-expert form (`train()`: the experts that were picked, each on its own
+tokens) and, where its E-fold work and memory fit, in its dense form (`eval()`: every expert on every token).
 """
 import argparse
 import json
@@ -45,7 +48,45 @@ def make_point(batch_size, seq_len, hidden_dim, num_experts, top_k, dtype=torch.
                 down_proj_bias=torch.ones(num_experts, hidden_dim, dtype=dtype, device=device))
 
 
-def run_point(batch_size, seq_len, hidden_dim, num_experts, top_k, iters=20, warmup=5, capacity="tokens", dtype=torch.float16):
+def time_torch_modules(p, tokens, hidden_dim, num_experts, iters, kernel_out):
+    """The torch experts module on the inputs of one point: milliseconds per call of its two forms and the distance of
+    its result from the kernel's."""
+    import types
+
+    from .reference import GptOssExperts
+    cfg = types.SimpleNamespace(hidden_size=hidden_dim, intermediate_size=hidden_dim, num_local_experts=num_experts)
+    with torch.device("meta"):
+        mod = GptOssExperts(cfg)
+    for name in ("gate_up_proj", "gate_up_proj_bias", "down_proj", "down_proj_bias"):
+        setattr(mod, name, torch.nn.Parameter(p[name], requires_grad=False))
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(iters):
+            out = fn()
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end) / iters, out
+
+    res = {}
+    with torch.no_grad():
+        mod.train()
+        ms, out = timed(lambda: mod(p["hidden"], p["router_indices"], p["routing_weights"]))
+        res["torch_per_expert_ms"] = round(ms, 4)
+        diff = (out.float() - kernel_out.float()).norm() / kernel_out.float().norm().clamp_min(1e-30)
+        res["rel_l2_vs_torch"] = float("%.3e" % float(diff))
+        del out
+        if num_experts * tokens * hidden_dim * 3 * 2 <= 24 << 30:   # the dense form holds [E, T, 3 * hidden] values
+            mod.eval()
+            res["torch_dense_ms"] = round(timed(lambda: mod(p["hidden"], p["router_indices"], p["routing_weights"]))[0], 4)
+    return res
+
+
+def run_point(batch_size, seq_len, hidden_dim, num_experts, top_k, iters=20, warmup=5, capacity="tokens", dtype=torch.float16,
+              torch_too=False):
     from . import experts
     p = make_point(batch_size, seq_len, hidden_dim, num_experts, top_k, dtype)
     tokens = batch_size * seq_len
@@ -66,7 +107,11 @@ def run_point(batch_size, seq_len, hidden_dim, num_experts, top_k, iters=20, war
     end.record()
     torch.cuda.synchronize()
     ms = start.elapsed_time(end) / iters
-    return dict(batch_size=batch_size, seq_len=seq_len, hidden_dim=hidden_dim, num_experts=num_experts, top_k=top_k,
+    extra = {}
+    if torch_too:
+        extra = time_torch_modules(p, tokens, hidden_dim, num_experts, max(3, iters // 4), out)
+        extra["speedup_vs_torch_per_expert"] = round(extra["torch_per_expert_ms"] / ms, 2)
+    return dict(**extra, batch_size=batch_size, seq_len=seq_len, hidden_dim=hidden_dim, num_experts=num_experts, top_k=top_k,
                 dtype=str(dtype).replace("torch.", ""), capacity=cap, kept_assignments=kept, ms=round(ms, 4),
                 tflops=round(kept * 6 * hidden_dim * hidden_dim / (ms * 1e-3) / 1e12, 2),
                 peak_extra_mib=round((torch.cuda.max_memory_allocated() - before) / 2 ** 20, 1),
@@ -79,10 +124,11 @@ def main(argv=None):
     ap.add_argument("--batches", default=",".join(str(b) for b in BATCH_SIZES))
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--capacity", choices=("seq", "tokens"), default="tokens")
+    ap.add_argument("--torch", action="store_true", help="also time the plain-torch experts module on the same inputs")
     a = ap.parse_args(argv)
     for ci in (int(c) for c in a.configs.split(",")):
         for b in (int(x) for x in a.batches.split(",")):
-            r = run_point(b, iters=a.iters, capacity=a.capacity, **CONFIGS[ci])
+            r = run_point(b, iters=a.iters, capacity=a.capacity, torch_too=a.torch, **CONFIGS[ci])
             r["config"] = ci
             print(json.dumps(r), flush=True)
             torch.cuda.empty_cache()
