@@ -38,3 +38,11 @@ def test_compare_reference_grid_point(gpu):
     assert r["memory_ratio"] > 1   # nothing here is padded to [E, C, *]
     r = compare_sweep.compare_point(64, iters=1, warmup=1, max_gflop=1.0, **sweep.CONFIGS[2])
     assert not r["compared"] and "kernel_vs_binned" not in r
+
+
+def test_sweep_point_against_the_torch_module(gpu):
+    """`--torch`: the plain-torch experts module on the same GPU and inputs, both forms timed, results close."""
+    from yamoe_amd import sweep
+    r = sweep.run_point(2, 64, 128, 8, 2, iters=4, warmup=1, torch_too=True)
+    assert r["finite"] and r["torch_per_expert_ms"] > 0 and r["torch_dense_ms"] > 0
+    assert r["rel_l2_vs_torch"] < 5e-3 and r["speedup_vs_torch_per_expert"] > 0
