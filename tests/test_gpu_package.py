@@ -31,6 +31,10 @@ grads = yamoe.experts_backward(gy.cuda(), *g, T, E, K)
 layer_out = yamoe.experts_autograd(*g, T, E, K, False) if hasattr(yamoe, 'experts_autograd') else out
 torch.cuda.synchronize()
 assert torch.equal(layer_out, out)
+# the torch baselines under the reference's names (torch-ext/yamoe/__init__.py:3-4, 29-31)
+ref = yamoe.vendored.yamoe_ref.binned_experts_ref(*[t.float() if t.is_floating_point() else t for t in g], T)
+assert (ref - out.float()).norm() / ref.norm() < 1e-2
+assert yamoe.reference.GptOssExperts is yamoe.gpt_oss_mlp.GptOssExperts
 torch.save(dict(inputs=d, gy=gy, out=out.cpu(), grads=[t.cpu() for t in grads], file=yamoe.__file__), sys.argv[2])
 print('child ok')
 """ % (KEYS,)

@@ -15,7 +15,8 @@ import shutil
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-MODULES = ("__init__.py", "_ops.py", "_cabi.py", "layers.py", "workloads.py", "sweep.py")
+MODULES = ("__init__.py", "_ops.py", "_cabi.py", "layers.py", "workloads.py", "sweep.py", "torch_baseline.py", "reference.py",
+           "vendored/__init__.py", "vendored/yamoe_ref.py", "vendored/gpt_oss_mlp.py")
 LIBS = ("libyamoe_hip.so", "_yamoe_amd_ops.so")
 
 BUILD_TOML = """[general]
@@ -53,6 +54,7 @@ def package(out_dir):
     dst = os.path.join(out_dir, "build", variant_name(), "yamoe")
     os.makedirs(dst, exist_ok=True)
     for name in MODULES + LIBS:
+        os.makedirs(os.path.dirname(os.path.join(dst, name)), exist_ok=True)
         shutil.copy2(os.path.join(HERE, name), os.path.join(dst, name))
     csrc = sorted(f for f in os.listdir(os.path.join(HERE, "csrc")) if f.endswith((".hip", ".h")))
     with open(os.path.join(out_dir, "build.toml"), "w") as f:
